@@ -1,0 +1,229 @@
+// C-ABI dispatcher: argument validation (host only), regime selection by activation-row count, launches.
+// Replaces the host launcher swiglu_fwd<TA,TB,TC> (swiglu.cu:397-525) and the convenience op's shape
+// derivation (swiglu.cu:538-553); the public contract is include/fsw.h.
+#include <hip/hip_runtime.h>
+#include <string.h>
+
+#include "fsw.h"
+#include "fsw_internal.h"
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+int g_forced_variant[2] = {-1, -1};  // family 0 = gate/up, 1 = down
+
+constexpr int VARIANT_SKINNY = 100;          // id of the weight-streaming kernel in fsw_set_variant
+constexpr int64_t MAX_DIM = 1LL << 30;       // every size is cast to int inside the kernels
+constexpr int64_t MAX_LD = 1LL << 21;        // keeps tile-relative byte offsets below 2^31
+
+bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+// gfx950 check, cached per device ordinal.
+int check_device() {
+  static int ok_mask[64] = {0};  // 0 unknown, 1 ok, 2 not gfx950
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    g_last_hip_error = (int)e;
+    return FSW_E_DEVICE;
+  }
+  if (dev < 0 || dev >= 64) return FSW_E_DEVICE;
+  if (ok_mask[dev] == 0) {
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) {
+      g_last_hip_error = (int)e;
+      return FSW_E_DEVICE;
+    }
+    ok_mask[dev] = (strncmp(prop.gcnArchName, "gfx950", 6) == 0) ? 1 : 2;
+  }
+  return ok_mask[dev] == 1 ? FSW_OK : FSW_E_DEVICE;
+}
+
+// Variant choice for the tiled kernels: the widest tile whose activation-row extent is not mostly padding,
+// stepping down to 128x128 when a 256-wide grid would leave most of the 256 CUs idle.
+int pick_tiled(int64_t m, int64_t np) {
+  if (m <= 32) return 4;   // 256 x 32
+  if (m <= 64) return 3;   // 256 x 64
+  if (m <= 128) return 1;  // 256 x 128
+  const int64_t tiles256 = ((np + 255) / 256) * ((m + 255) / 256);
+  if (tiles256 < 192) return 2;  // 128 x 128
+  return 0;                      // 256 x 256
+}
+
+int resolve_variant(int family, int64_t m, int64_t np) {
+  const int forced = g_forced_variant[family];
+  if (forced >= 0) return forced;
+  return pick_tiled(m, np);
+}
+
+int finish(hipError_t e) {
+  if (e != hipSuccess) {
+    g_last_hip_error = (int)e;
+    return FSW_E_LAUNCH;
+  }
+  return FSW_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fsw_version(void) { return 1000; }
+
+const char* fsw_strerror(int code) {
+  switch (code) {
+    case FSW_OK: return "ok";
+    case FSW_E_NULL: return "fsw: a required pointer is NULL";
+    case FSW_E_DTYPE: return "fsw: unsupported element type (expected bf16 or fp16)";
+    case FSW_E_SHAPE: return "fsw: bad shape (negative size, odd N, or size out of range)";
+    case FSW_E_LD: return "fsw: leading dimension smaller than the row it strides";
+    case FSW_E_ALIGN: return "fsw: K/FF and leading dimensions must be multiples of 8 and inputs 16-byte aligned";
+    case FSW_E_WORKSPACE: return "fsw: workspace missing or too small";
+    case FSW_E_LAUNCH: return "fsw: the HIP runtime rejected the kernel launch";
+    case FSW_E_DEVICE: return "fsw: the current device is not a gfx950 GPU";
+    case FSW_E_VARIANT: return "fsw: unknown kernel variant";
+    default: return "fsw: unknown error code";
+  }
+}
+
+int fsw_last_hip_error(void) { return g_last_hip_error; }
+
+int fsw_set_variant(int family, int variant) {
+  if (family < 0 || family > 1) return FSW_E_VARIANT;
+  if (variant >= 0 && variant != VARIANT_SKINNY && variant >= fsw::tiled_variant_count()) return FSW_E_VARIANT;
+  g_forced_variant[family] = variant < 0 ? -1 : variant;
+  return FSW_OK;
+}
+
+const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, int64_t K_or_FF) {
+  (void)dtype;
+  (void)K_or_FF;
+  if (family < 0 || family > 1) return "invalid";
+  const int v = resolve_variant(family, M, N_or_D);
+  if (v == VARIANT_SKINNY) return "skinny";
+  return fsw::tiled_variant(v).name;
+}
+
+int fsw_validate_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13,
+                        int64_t ldw, const void* H, int64_t ldh) {
+  if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
+  if (M < 0 || N < 0 || K < 0 || (N & 1)) return FSW_E_SHAPE;
+  if (M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return FSW_E_SHAPE;
+  if (M == 0 || N == 0) return FSW_OK;  // nothing to read or write
+  if (!X || !W13 || !H) return FSW_E_NULL;
+  if (ldx < K || ldw < K || ldh < N / 2) return FSW_E_LD;
+  if (ldx > MAX_LD || ldw > MAX_LD || ldh > MAX_DIM) return FSW_E_SHAPE;
+  if ((K & 7) || (ldx & 7) || (ldw & 7)) return FSW_E_ALIGN;
+  if (!aligned16(X) || !aligned16(W13) || (((uintptr_t)H) & 1)) return FSW_E_ALIGN;
+  return FSW_OK;
+}
+
+int fsw_validate_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t ldh, const void* W2,
+                      int64_t ldw2, const void* Y, int64_t ldy) {
+  if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
+  if (M < 0 || D < 0 || FF < 0) return FSW_E_SHAPE;
+  if (M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM) return FSW_E_SHAPE;
+  if (M == 0 || D == 0) return FSW_OK;
+  if (!H || !W2 || !Y) return FSW_E_NULL;
+  if (ldh < FF || ldw2 < FF || ldy < D) return FSW_E_LD;
+  if (ldh > MAX_LD || ldw2 > MAX_LD || ldy > MAX_DIM) return FSW_E_SHAPE;
+  if ((FF & 7) || (ldh & 7) || (ldw2 & 7)) return FSW_E_ALIGN;
+  if (!aligned16(H) || !aligned16(W2) || (((uintptr_t)Y) & 1)) return FSW_E_ALIGN;
+  return FSW_OK;
+}
+
+int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13, int64_t ldw,
+               void* H, int64_t ldh, void* stream) {
+  const int rc = fsw_validate_gateup(dtype, M, N, K, X, ldx, W13, ldw, H, ldh);
+  if (rc != FSW_OK) return rc;
+  if (M == 0 || N == 0) return FSW_OK;
+  const int drc = check_device();
+  if (drc != FSW_OK) return drc;
+  fsw::GemmArgs a;
+  a.P = W13;
+  a.Q = X;
+  a.O = H;
+  a.ldp = ldw;
+  a.ldq = ldx;
+  a.ldo = ldh;
+  a.np = (int)N;
+  a.nq = (int)M;
+  a.k = (int)K;
+  const int v = resolve_variant(0, M, N);
+  if (v == VARIANT_SKINNY) return FSW_E_VARIANT;
+  return finish(fsw::launch_tiled(v, dtype, true, a, (hipStream_t)stream));
+}
+
+size_t fsw_down_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
+  (void)dtype;
+  (void)M;
+  (void)D;
+  (void)FF;
+  return 0;
+}
+
+int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t ldh, const void* W2, int64_t ldw2,
+             void* Y, int64_t ldy, void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = fsw_validate_down(dtype, M, D, FF, H, ldh, W2, ldw2, Y, ldy);
+  if (rc != FSW_OK) return rc;
+  if (M == 0 || D == 0) return FSW_OK;
+  const size_t need = fsw_down_workspace_bytes(dtype, M, D, FF);
+  if (need > 0 && (!workspace || workspace_bytes < need)) return FSW_E_WORKSPACE;
+  const int drc = check_device();
+  if (drc != FSW_OK) return drc;
+  fsw::GemmArgs a;
+  a.P = W2;
+  a.Q = H;
+  a.O = Y;
+  a.ldp = ldw2;
+  a.ldq = ldh;
+  a.ldo = ldy;
+  a.np = (int)D;
+  a.nq = (int)M;
+  a.k = (int)FF;
+  const int v = resolve_variant(1, M, D);
+  if (v == VARIANT_SKINNY) return FSW_E_VARIANT;
+  return finish(fsw::launch_tiled(v, dtype, false, a, (hipStream_t)stream));
+}
+
+static size_t h_bytes(int64_t M, int64_t FF) {
+  const size_t raw = (size_t)M * (size_t)FF * 2;
+  return (raw + 255) & ~(size_t)255;
+}
+
+size_t fsw_mlp_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
+  if (M <= 0 || D <= 0 || FF <= 0) return 0;
+  return h_bytes(M, FF) + fsw_down_workspace_bytes(dtype, M, D, FF);
+}
+
+int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t ldx, const void* W13, int64_t ldw13,
+            const void* W2, int64_t ldw2, void* Y, int64_t ldy, void* workspace, size_t workspace_bytes,
+            void* stream) {
+  if (M < 0 || D < 0 || FF < 0 || FF > MAX_DIM / 2) return FSW_E_SHAPE;
+  const size_t need = fsw_mlp_workspace_bytes(dtype, M, D, FF);
+  if (need > 0 && (!workspace || workspace_bytes < need)) return FSW_E_WORKSPACE;
+  if (need > 0 && !aligned16(workspace)) return FSW_E_ALIGN;
+  if (FF == 0) {
+    // empty inner dimension: Y = 0, nothing else is read
+    if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
+    if (M == 0 || D == 0) return FSW_OK;
+    if (!Y) return FSW_E_NULL;
+    if (ldy < D) return FSW_E_LD;
+    hipError_t e = hipMemset2DAsync(Y, (size_t)ldy * 2, 0, (size_t)D * 2, (size_t)M, (hipStream_t)stream);
+    return finish(e);
+  }
+  void* Hbuf = workspace;
+  // validate both halves before launching either, so a bad down-projection argument leaves nothing enqueued
+  int rc = fsw_validate_gateup(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF);
+  if (rc != FSW_OK) return rc;
+  rc = fsw_validate_down(dtype, M, D, FF, Hbuf, FF, W2, ldw2, Y, ldy);
+  if (rc != FSW_OK) return rc;
+  if (M == 0 || D == 0) return FSW_OK;
+  rc = fsw_gateup(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF, stream);
+  if (rc != FSW_OK) return rc;
+  unsigned char* ws2 = (unsigned char*)workspace + h_bytes(M, FF);
+  return fsw_down(dtype, M, D, FF, Hbuf, FF, W2, ldw2, Y, ldy, ws2, workspace_bytes - h_bytes(M, FF), stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,39 @@
+// Internal launcher interface between the C-ABI dispatcher (fsw_api.hip) and the kernel translation units.
+// Nothing here is exported; the public surface is include/fsw.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fsw {
+
+// One TN GEMM problem in "weight rows x activation rows" form.
+//   P: weight operand, [np, k] row-major (W13 for the gated kernel, W2 for the down kernel)
+//   Q: activation operand, [nq, k] row-major (X or H)
+//   O: output, [nq, np/2] (gated) or [nq, np] (plain), row stride ldo
+struct GemmArgs {
+  const void* P;
+  const void* Q;
+  void* O;
+  long long ldp, ldq, ldo;  // elements
+  int np, nq, k;
+};
+
+// Tiled LDS/MFMA kernels (kernels_tiled.hip). `variant` indexes tiled_variant_table().
+struct TiledVariant {
+  const char* name;
+  int bp, bq;        // workgroup tile: weight rows x activation rows
+  int threads;
+};
+int tiled_variant_count();
+const TiledVariant& tiled_variant(int variant);
+hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
+
+// Weight-streaming kernels for M <= 16 activation rows (kernels_skinny.hip).
+struct SkinnyPlan {
+  int splits;              // K partitions per weight-row tile across workgroups (1 = no scratch needed)
+  size_t workspace_bytes;  // fp32 partials + arrival counters
+};
+SkinnyPlan skinny_plan(bool gated, int np, int nq, int k);
+hipError_t launch_skinny(int dtype, bool gated, const GemmArgs& a, void* workspace, hipStream_t stream);
+
+}  // namespace fsw

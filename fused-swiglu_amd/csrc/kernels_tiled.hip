@@ -1,0 +1,286 @@
+// LDS-tiled MFMA kernels for the compute-bound (prefill) regime on gfx950.
+//
+// One kernel template covers both GEMMs of the MLP forward:
+//   GATED : H[m, j] = up * silu(gate), up = X[m,:].W13[2j,:], gate = X[m,:].W13[2j+1,:]
+//           (the computation of swiglu.cu:111-394: main loop :290-343, gating epilogue :345-393)
+//   plain : Y[m, n] = H[m,:].W2[n,:]   (no counterpart in the reference)
+//
+// Orientation. The MFMA "A" operand (rows of the 32x32 result) is fed with WEIGHT rows and the "B" operand
+// (columns of the result) with ACTIVATION rows, so an accumulator lane owns one activation row m and runs of 4
+// consecutive output features. That makes the stores 8-byte vectors along the contiguous dimension of the
+// output, and, for the gated kernel, lets the de-interleave of W13 happen while the tile is copied into LDS:
+// LDS rows [0, BP/2) receive the even ("up") rows of the weight tile and rows [BP/2, BP) the odd ("gate")
+// rows. A wave then runs two accumulator sets over the same activation fragments, and up/gate of one (m, j)
+// land in the same lane and register index: the gating is plain per-lane fp32 math, no cross-lane traffic.
+//
+// LDS layout. Each operand tile is [rows][64 elements] = 128 bytes per row, eight 16-byte chunks; chunk c of
+// row r is stored at chunk position c ^ (r & 7). A wave's ds_read_b128 for an MFMA operand touches 32
+// consecutive rows at one logical chunk (x2 for the two K halves), so any 8 consecutive lanes cover all 32
+// banks exactly once; the global->LDS copy writes whole 128-byte rows per 8 lanes. Both are conflict-free.
+#include "fsw_internal.h"
+#include "fsw_device.h"
+
+namespace fsw {
+
+template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
+__global__ void __launch_bounds__(WP* WQ * 64)
+tiled_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
+  constexpr int NT = WP * WQ * 64;
+  constexpr int BP = WP * FP * 32;  // weight rows per workgroup tile
+  constexpr int BQ = WQ * FQ * 32;  // activation rows per workgroup tile
+  constexpr int BK = 64;            // K elements per LDS stage
+  constexpr int ROWB = BK * 2;      // bytes per LDS row
+  constexpr int RSTEP = NT / 8;     // row distance between a thread's successive 16-byte copies
+  constexpr int LP = BP / RSTEP;    // copies per thread per stage, weight tile
+  constexpr int LQ = BQ / RSTEP;    // copies per thread per stage, activation tile
+  constexpr int STAGE = (BP + BQ) * ROWB;
+  static_assert(BP % RSTEP == 0 && BQ % RSTEP == 0 && RSTEP % 8 == 0, "copy mapping");
+  static_assert(!GATED || (FP % 2 == 0), "gated kernel pairs fragments");
+  static_assert(2 * STAGE <= 160 * 1024, "LDS budget of a gfx950 CU");
+
+  __shared__ __align__(16) unsigned char lds[2 * STAGE];
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = t >> 6;
+  const int wq = wave % WQ;
+  const int wp = wave / WQ;
+  const int l32 = lane & 31;
+  const int hi = lane >> 5;
+
+  int tp, tq;
+  tile_coords(blockIdx.x, tiles_p, tiles_q, group, tp, tq);
+  const int p0 = tp * BP;
+  const int q0 = tq * BQ;
+
+  // ---- global -> register copy mapping: thread copies chunk `c` of rows rb, rb+RSTEP, ...
+  const int c = t & 7;
+  const int rb = t >> 3;
+  const unsigned char* pbase = (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
+  const unsigned char* qbase = (const unsigned char*)a.Q + (long long)q0 * a.ldq * 2;
+  const __amdgpu_buffer_rsrc_t prs = make_rsrc(pbase, ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
+  const __amdgpu_buffer_rsrc_t qrs = make_rsrc(qbase, ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2);
+
+  unsigned poff[LP], qoff[LQ];
+#pragma unroll
+  for (int i = 0; i < LP; ++i) {
+    const int r = rb + i * RSTEP;
+    const int grow = GATED ? (r < BP / 2 ? 2 * r : 2 * (r - BP / 2) + 1) : r;
+    poff[i] = (unsigned)grow * (unsigned)a.ldp * 2u + (unsigned)c * 16u;
+  }
+#pragma unroll
+  for (int i = 0; i < LQ; ++i) {
+    const int r = rb + i * RSTEP;
+    qoff[i] = (unsigned)r * (unsigned)a.ldq * 2u + (unsigned)c * 16u;
+  }
+  // LDS byte address of this thread's first copy; later copies add i * RSTEP * ROWB (RSTEP % 8 == 0 keeps r & 7).
+  const unsigned wr_p = (unsigned)rb * ROWB + (unsigned)((c ^ (rb & 7)) * 16);
+  const unsigned wr_q = (unsigned)BP * ROWB + wr_p;
+
+  // ---- LDS -> MFMA fragment read mapping
+  unsigned xo[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) xo[ks] = (unsigned)((((ks << 1) | hi) ^ (lane & 7)) * 16);
+  const unsigned rd_p = (unsigned)((GATED ? wp * (FP / 2) * 32 : wp * FP * 32) + l32) * ROWB;
+  const unsigned rd_q = (unsigned)(BP + wq * FQ * 32 + l32) * ROWB;
+  auto p_frag_off = [](int f) -> unsigned {
+    if (GATED) return (unsigned)((f < FP / 2 ? f * 32 : BP / 2 + (f - FP / 2) * 32) * ROWB);
+    return (unsigned)(f * 32 * ROWB);
+  };
+
+  f32x16 acc[FP][FQ];
+#pragma unroll
+  for (int f = 0; f < FP; ++f)
+#pragma unroll
+    for (int g = 0; g < FQ; ++g)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[f][g][i] = 0.0f;
+
+  u32x4 sp[LP], sq[LQ];
+  const int nkt = (a.k + BK - 1) / BK;
+
+  // Copies for K tile `kt`; tiles at or beyond K read as zero (hardware bounds check), so the pipeline below
+  // can prefetch past the end without branching.
+  auto g_load = [&](int kt) {
+    const unsigned kb = (unsigned)kt * (BK * 2);
+    const bool in = (kt * BK + c * 8) < a.k;
+#pragma unroll
+    for (int i = 0; i < LP; ++i) sp[i] = buf_load16(prs, in ? poff[i] + kb : OOB_OFFSET);
+#pragma unroll
+    for (int i = 0; i < LQ; ++i) sq[i] = buf_load16(qrs, in ? qoff[i] + kb : OOB_OFFSET);
+  };
+  auto s_store = [&](int stage) {
+    unsigned char* base = lds + stage * STAGE;
+#pragma unroll
+    for (int i = 0; i < LP; ++i) *(u32x4*)(base + wr_p + i * RSTEP * ROWB) = sp[i];
+#pragma unroll
+    for (int i = 0; i < LQ; ++i) *(u32x4*)(base + wr_q + i * RSTEP * ROWB) = sq[i];
+  };
+
+  u32x4 pf[2][FP], qf[2][FQ];
+  // Fragment reads for K step `ks` of LDS stage `stage`, issued in the order the MFMAs consume them.
+  auto f_read = [&](int fb, int stage, int ks) {
+    const unsigned char* base = lds + stage * STAGE;
+    pf[fb][0] = *(const u32x4*)(base + rd_p + p_frag_off(0) + xo[ks]);
+#pragma unroll
+    for (int g = 0; g < FQ; ++g) qf[fb][g] = *(const u32x4*)(base + rd_q + g * 32 * ROWB + xo[ks]);
+#pragma unroll
+    for (int f = 1; f < FP; ++f) pf[fb][f] = *(const u32x4*)(base + rd_p + p_frag_off(f) + xo[ks]);
+  };
+  auto mma = [&](int fb, int f_lo, int f_hi) {
+#pragma unroll
+    for (int f = f_lo; f < f_hi; ++f)
+#pragma unroll
+      for (int g = 0; g < FQ; ++g) acc[f][g] = E::mfma32(pf[fb][f], qf[fb][g], acc[f][g]);
+  };
+
+  // Software pipeline, one barrier per K tile of 64:
+  //   K steps 0..2 : MFMAs of step s overlap the LDS fragment reads of step s+1 (same stage);
+  //   K step 3, a  : first half of the MFMAs overlaps the ds_writes of tile kt+1 (in registers since the
+  //                  previous iteration) into the other stage; barrier;
+  //   K step 3, b  : second half of the MFMAs overlaps the fragment reads of step 0 of tile kt+1 and the
+  //                  global loads of tile kt+2.
+  // The other stage is free for writing during the whole iteration: every wave finished its reads of it
+  // before the barrier of the previous iteration (they are issued in steps 0..2 and in 3b of the one before).
+  g_load(0);
+  s_store(0);
+  g_load(1);
+  __syncthreads();
+  f_read(0, 0, 0);
+
+  // Issue-order hints for the machine scheduler (masks: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS read,
+  // 0x200 LDS write). Without them the compiler sinks every fragment read next to its first use and the
+  // LDS latency is exposed once per K step.
+  constexpr int NM = FP * FQ;                      // MFMAs per K step
+  constexpr int NR = FP + FQ;                      // fragment reads per K step
+  constexpr int HF = FP / 2 > 0 ? FP / 2 : 1;      // fragments in the first half of step 3
+  constexpr int MPR = NM / NR > 0 ? NM / NR : 1;   // MFMAs per fragment read
+  auto hint_reads = [&]() {
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+  };
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int cur = kt & 1;
+    // K step 0
+    f_read(1, cur, 1);
+    mma(0, 0, FP);
+    hint_reads();
+    // K step 1
+    f_read(0, cur, 2);
+    mma(1, 0, FP);
+    hint_reads();
+    // K step 2
+    f_read(1, cur, 3);
+    mma(0, 0, FP);
+    hint_reads();
+    // K step 3a
+    mma(1, 0, HF);
+    s_store(cur ^ 1);
+#pragma unroll
+    for (int i = 0; i < HF * FQ; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x200, (LP + LQ + HF * FQ - 1) / (HF * FQ), 0);
+    }
+    __syncthreads();
+    // K step 3b
+    f_read(0, cur ^ 1, 0);
+    g_load(kt + 2);
+    mma(1, HF, FP);
+#pragma unroll
+    for (int i = 0; i < (FP - HF) * FQ; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x100, (NR + (FP - HF) * FQ - 1) / ((FP - HF) * FQ), 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, (LP + LQ + (FP - HF) * FQ - 1) / ((FP - HF) * FQ), 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+  }
+
+  // ---- epilogue: lane owns activation row m = l32 of each Q fragment and, per group of 4 accumulator
+  // registers, 4 consecutive output features: feature = 8 * (i / 4) + 4 * hi + (i % 4) within the fragment.
+  unsigned short* O = (unsigned short*)a.O;
+  const int nout = GATED ? a.np / 2 : a.np;
+  const bool vec_ok = ((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 7) == 0);
+  constexpr int FO = GATED ? FP / 2 : FP;
+#pragma unroll
+  for (int g = 0; g < FQ; ++g) {
+    const int m = q0 + (wq * FQ + g) * 32 + l32;
+    if (m >= a.nq) continue;
+    unsigned short* orow = O + (long long)m * a.ldo;
+#pragma unroll
+    for (int f = 0; f < FO; ++f) {
+      const int nb = (GATED ? p0 / 2 + (wp * FO + f) * 32 : p0 + (wp * FO + f) * 32) + hi * 4;
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (GATED) {
+            v[e] = acc[f][g][i4 * 4 + e] * silu_f32(acc[f + FO][g][i4 * 4 + e]);
+          } else {
+            v[e] = acc[f][g][i4 * 4 + e];
+          }
+        }
+        const int n = nb + i4 * 8;
+        if (vec_ok && n + 3 < nout) {
+          u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
+          *(u32x2*)(orow + n) = pk;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < nout) orow[n + e] = E::cvt1(v[e]);
+        }
+      }
+    }
+  }
+}
+
+// ---- variant table ------------------------------------------------------------------------------------
+namespace {
+
+const TiledVariant kVariants[] = {
+    {"tiled_256x256", 256, 256, 256},  // large-M prefill: 4 waves, 128x128 accumulators per wave
+    {"tiled_256x128", 256, 128, 256},
+    {"tiled_128x128", 128, 128, 256},
+    {"tiled_256x64", 256, 64, 256},
+    {"tiled_256x32", 256, 32, 256},
+};
+
+template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
+hipError_t launch_one(const GemmArgs& a, hipStream_t stream) {
+  constexpr int BP = WP * FP * 32, BQ = WQ * FQ * 32;
+  const int tiles_p = (a.np + BP - 1) / BP;
+  const int tiles_q = (a.nq + BQ - 1) / BQ;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  const int group = 4;
+  hipLaunchKernelGGL((tiled_kernel<E, GATED, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)), dim3(WP * WQ * 64), 0,
+                     stream, a, tiles_p, tiles_q, group);
+  return hipGetLastError();
+}
+
+template <class E, bool GATED>
+hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
+  switch (variant) {
+    case 0: return launch_one<E, GATED, 2, 2, 4, 4>(a, stream);
+    case 1: return launch_one<E, GATED, 2, 2, 4, 2>(a, stream);
+    case 2: return launch_one<E, GATED, 2, 2, 2, 2>(a, stream);
+    case 3: return launch_one<E, GATED, 4, 1, 2, 2>(a, stream);
+    case 4: return launch_one<E, GATED, 4, 1, 2, 1>(a, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
+int tiled_variant_count() { return (int)(sizeof(kVariants) / sizeof(kVariants[0])); }
+const TiledVariant& tiled_variant(int variant) { return kVariants[variant]; }
+
+hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, hipStream_t stream) {
+  if (dtype == 0) {
+    return gated ? launch_variant<Bf16, true>(variant, a, stream) : launch_variant<Bf16, false>(variant, a, stream);
+  }
+  return gated ? launch_variant<Fp16, true>(variant, a, stream) : launch_variant<Fp16, false>(variant, a, stream);
+}
+
+}  // namespace fsw

@@ -1,0 +1,127 @@
+/*
+ * fsw.h — C ABI of the MI355X (gfx950) fused SwiGLU MLP forward.
+ *
+ * The reference (bit-ml/Fused-SwiGLU) has no C ABI: its internal boundary is the C++ template
+ * `swiglu_fwd<TA,TB,TC>` declared at csrc/torch_bindings.cpp:16-27 and defined at
+ * csrc/SwiGLU/swiglu.cu:397-525, plus the convenience op `fused_swiglu_bf16` (swiglu.cu:538-553).
+ * The entry points below are what a foreign-function binding for that path binds instead; the
+ * PyTorch operator surface (torch_bindings.cpp:31-50) is rebuilt on top of them.
+ *
+ * Conventions (all entry points):
+ *   - every data pointer is a DEVICE pointer owned by the caller; nothing is allocated or freed here;
+ *   - leading dimensions (ld*) are in ELEMENTS, inner (K) stride is 1 as in swiglu.cu:411-414;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); launches are
+ *     asynchronous, nothing here synchronises;
+ *   - the return value is FSW_OK (0) or a negative FSW_E_* code; nothing throws or aborts;
+ *   - the fsw_validate_* functions touch no GPU API and can be called on a machine without one.
+ *
+ * Weight formats (identical to the reference's):
+ *   W13 [N = 2*ff, K] row-major, K-contiguous, rows interleaved: row 2j   = "up"  (linear) operand,
+ *                                                                row 2j+1 = "gate" (SiLU) operand
+ *       (swiglu.cu:380-381, numeric_tests.py:41-43);
+ *   W2  [D, FF] row-major, FF-contiguous (the transpose of the mathematical Wd[FF, D]).
+ */
+#ifndef FSW_H
+#define FSW_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* every entry point below is exported; everything else in the library has hidden visibility */
+#define FSW_API __attribute__((visibility("default")))
+
+/* element types */
+#define FSW_BF16 0
+#define FSW_FP16 1
+
+/* error codes */
+#define FSW_OK            0
+#define FSW_E_NULL       -1   /* a required pointer is NULL */
+#define FSW_E_DTYPE      -2   /* dtype is not FSW_BF16 / FSW_FP16 */
+#define FSW_E_SHAPE      -3   /* negative size, odd N, or a size beyond the supported range */
+#define FSW_E_LD         -4   /* leading dimension smaller than the row it strides */
+#define FSW_E_ALIGN      -5   /* K (or FF), a leading dimension or a pointer breaks the 16-byte rule */
+#define FSW_E_WORKSPACE  -6   /* workspace missing or smaller than fsw_*_workspace_bytes() */
+#define FSW_E_LAUNCH     -7   /* the HIP runtime rejected a launch (see fsw_last_hip_error) */
+#define FSW_E_DEVICE     -8   /* the current device is not a gfx950 GPU */
+#define FSW_E_VARIANT    -9   /* unknown kernel variant requested through fsw_set_variant */
+
+/*
+ * Host-only argument validation of fsw_gateup (replaces the dtype TORCH_CHECKs of swiglu.cu:475-480 and adds
+ * the shape/stride checks the reference leaves out). Rules: M >= 0; N >= 0 and even; K >= 0 and K % 8 == 0
+ * (16-byte vectors; the reference needs K % 32 == 0, swiglu.cu:220-230); ldx >= K, ldw >= K, ldh >= N/2;
+ * ldx % 8 == 0 and ldw % 8 == 0; pointers non-NULL and X, W13 16-byte aligned when the problem is non-empty.
+ */
+FSW_API int fsw_validate_gateup(int dtype, int64_t M, int64_t N, int64_t K,
+                        const void* X, int64_t ldx, const void* W13, int64_t ldw,
+                        const void* H, int64_t ldh);
+
+/*
+ * H[M, N/2] = up * silu(gate) with up = X @ W13[0::2].T, gate = X @ W13[1::2].T; fp32 accumulation,
+ * fp32 gating, ONE round-to-nearest-even to the element type on store.
+ * Replaces swiglu_fwd<bf16,bf16,bf16> (swiglu.cu:397-525; kernel swiglu.cu:103-394). N is the FULL 2*ff as in
+ * the reference; ldh is the row stride of H itself (the reference's operator passes ldC/2, swiglu.cu:414).
+ */
+FSW_API int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K,
+               const void* X, int64_t ldx, const void* W13, int64_t ldw,
+               void* H, int64_t ldh, void* stream);
+
+/* Host-only validation of fsw_down: M, D, FF >= 0; FF % 8 == 0; ldh >= FF, ldw2 >= FF, ldy >= D;
+ * ldh % 8 == 0, ldw2 % 8 == 0; H, W2 16-byte aligned. */
+FSW_API int fsw_validate_down(int dtype, int64_t M, int64_t D, int64_t FF,
+                      const void* H, int64_t ldh, const void* W2, int64_t ldw2,
+                      const void* Y, int64_t ldy);
+
+/* Bytes of device scratch fsw_down needs for this shape (fp32 split-K partials in the small-M regime;
+ * 0 when the shape runs without scratch). No counterpart in the reference, which has no down projection. */
+FSW_API size_t fsw_down_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF);
+
+/*
+ * Y[M, D] = H[M, FF] @ W2[D, FF].T, fp32 accumulation, one RNE rounding on store.
+ * No counterpart in the reference (its op ends at H, swiglu.cu:538-553); it is the `@ Wd` step of the
+ * full MLP forward (silu(X@Wg) * (X@Wu)) @ Wd.
+ */
+FSW_API int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF,
+             const void* H, int64_t ldh, const void* W2, int64_t ldw2,
+             void* Y, int64_t ldy,
+             void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes of device scratch fsw_mlp needs: the H[M, FF] intermediate plus fsw_down's scratch. */
+FSW_API size_t fsw_mlp_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF);
+
+/*
+ * Whole forward: Y[M, D] = (silu(X @ Wg) * (X @ Wu)) @ Wd as fsw_gateup followed by fsw_down on the same
+ * stream, with H held in `workspace`. X is [M, D]; W13 is [2*FF, D]; W2 is [D, FF].
+ */
+FSW_API int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF,
+            const void* X, int64_t ldx, const void* W13, int64_t ldw13,
+            const void* W2, int64_t ldw2, void* Y, int64_t ldy,
+            void* workspace, size_t workspace_bytes, void* stream);
+
+/* Text for an FSW_E_* code (static storage, never NULL). */
+FSW_API const char* fsw_strerror(int code);
+
+/* The hipError_t (as int) of the most recent failed launch on the calling thread, 0 if none. */
+FSW_API int fsw_last_hip_error(void);
+
+/* ABI version: major * 1000 + minor. */
+FSW_API int fsw_version(void);
+
+/*
+ * Kernel-selection override for tuning and tests. family: 0 = gate/up, 1 = down.
+ * variant < 0 restores the automatic choice by shape. Returns FSW_E_VARIANT for unknown ids.
+ * Process-wide and not thread-safe against concurrent launches.
+ */
+FSW_API int fsw_set_variant(int family, int variant);
+
+/* Name of the kernel variant the dispatcher picks for this shape (static storage). */
+FSW_API const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, int64_t K_or_FF);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FSW_H */

@@ -1,0 +1,179 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports everything include/fsw.h declares,
+argument validation returns the documented codes before any HIP call, the packers follow the reference's
+row interleave, and the operator surface matches csrc/torch_bindings.cpp:31-50 of the reference."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import fsw_weights
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fsw.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"FSW_API\s+[\w\s\*]+?\b(fsw_\w+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol(capi):
+    names = declared_symbols()
+    assert len(names) >= 12 and len(set(names)) == len(names)
+    raw = ctypes.CDLL(capi.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), "libfsw_hip.so does not export %s" % n
+    # the ctypes prototypes cover exactly the header
+    assert sorted(capi.PROTOTYPES) == sorted(names)
+    assert capi.lib().fsw_version() >= 1000
+
+
+def test_strerror_covers_all_codes(capi):
+    seen = set()
+    for code in range(0, -10, -1):
+        s = capi.strerror(code)
+        assert s and s not in seen
+        seen.add(s)
+    assert "unknown" in capi.strerror(-99)
+
+
+def _v_gateup(capi, dtype=0, M=4, N=8, K=16, X=0x1000, ldx=None, W=0x2000, ldw=None, H=0x3000, ldh=None):
+    return capi.lib().fsw_validate_gateup(dtype, M, N, K, X, K if ldx is None else ldx, W, K if ldw is None else ldw,
+                                          H, N // 2 if ldh is None else ldh)
+
+
+def test_validate_gateup_codes(capi):
+    assert _v_gateup(capi) == capi.OK
+    assert _v_gateup(capi, dtype=1) == capi.OK
+    assert _v_gateup(capi, dtype=2) == capi.E_DTYPE
+    assert _v_gateup(capi, M=-1) == capi.E_SHAPE
+    assert _v_gateup(capi, N=7) == capi.E_SHAPE          # odd N: rows come in (up, gate) pairs
+    assert _v_gateup(capi, M=2 ** 31) == capi.E_SHAPE
+    assert _v_gateup(capi, K=12) == capi.E_ALIGN         # K % 8
+    assert _v_gateup(capi, ldx=8) == capi.E_LD
+    assert _v_gateup(capi, ldw=8) == capi.E_LD
+    assert _v_gateup(capi, ldh=3) == capi.E_LD
+    assert _v_gateup(capi, ldx=20) == capi.E_ALIGN       # ld % 8
+    assert _v_gateup(capi, X=0x1008) == capi.E_ALIGN     # 16-byte rule
+    assert _v_gateup(capi, W=0x2004) == capi.E_ALIGN
+    assert _v_gateup(capi, X=None) == capi.E_NULL
+    assert _v_gateup(capi, W=None) == capi.E_NULL
+    assert _v_gateup(capi, H=None) == capi.E_NULL
+    # empty problems need no pointers at all
+    assert _v_gateup(capi, M=0, X=None, W=None, H=None) == capi.OK
+    assert _v_gateup(capi, N=0, X=None, W=None, H=None) == capi.OK
+    # K = 0 is a valid (all-zero) product
+    assert _v_gateup(capi, K=0) == capi.OK
+
+
+def test_validate_down_codes(capi):
+    v = capi.lib().fsw_validate_down
+    assert v(0, 4, 8, 16, 0x1000, 16, 0x2000, 16, 0x3000, 8) == capi.OK
+    assert v(3, 4, 8, 16, 0x1000, 16, 0x2000, 16, 0x3000, 8) == capi.E_DTYPE
+    assert v(0, 4, 8, 12, 0x1000, 16, 0x2000, 16, 0x3000, 8) == capi.E_ALIGN
+    assert v(0, 4, 8, 16, 0x1000, 8, 0x2000, 16, 0x3000, 8) == capi.E_LD
+    assert v(0, 4, 8, 16, 0x1000, 16, 0x2000, 16, 0x3000, 4) == capi.E_LD
+    assert v(0, 4, 8, 16, None, 16, 0x2000, 16, 0x3000, 8) == capi.E_NULL
+    assert v(0, 4, -8, 16, 0x1000, 16, 0x2000, 16, 0x3000, 8) == capi.E_SHAPE
+    assert v(0, 0, 8, 16, None, 16, None, 16, None, 8) == capi.OK
+
+
+def test_entry_points_reject_bad_arguments_before_touching_the_gpu(capi):
+    L = capi.lib()
+    # these return from validation, so they are safe on a machine without a GPU
+    assert L.fsw_gateup(0, 4, 7, 16, 0x1000, 16, 0x2000, 16, 0x3000, 4, None) == capi.E_SHAPE
+    assert L.fsw_gateup(5, 4, 8, 16, 0x1000, 16, 0x2000, 16, 0x3000, 4, None) == capi.E_DTYPE
+    assert L.fsw_gateup(0, 0, 8, 16, None, 16, None, 16, None, 4, None) == capi.OK
+    assert L.fsw_down(0, 4, 8, 12, 0x1000, 16, 0x2000, 16, 0x3000, 8, None, 0, None) == capi.E_ALIGN
+    assert L.fsw_mlp(0, 4, 16, 8, 0x1000, 16, 0x2000, 16, 0x3000, 8, 0x4000, 16, None, 0, None) == capi.E_WORKSPACE
+    assert L.fsw_mlp_workspace_bytes(0, 4, 16, 8) >= 4 * 8 * 2
+    assert L.fsw_mlp_workspace_bytes(0, 0, 16, 8) == 0
+    assert L.fsw_set_variant(0, 12345) == capi.E_VARIANT
+    assert L.fsw_set_variant(7, 0) == capi.E_VARIANT
+    assert L.fsw_set_variant(0, -1) == capi.OK
+    with pytest.raises(capi.FswError) as ei:
+        capi.check(capi.E_ALIGN)
+    assert isinstance(ei.value, RuntimeError) and ei.value.code == capi.E_ALIGN
+
+
+def test_variant_choice_by_regime(capi):
+    name = lambda fam, M, n, k: capi.variant_name(fam, 0, M, n, k)
+    assert name(0, 8192, 28672, 4096) == "tiled_256x256"
+    assert name(1, 8192, 4096, 14336) == "tiled_256x256"
+    assert "256" in name(0, 4096, 22016, 4096)
+    assert name(0, 512, 5632, 1024) == "tiled_128x128"   # small problem: more, smaller tiles
+
+
+def test_packers_follow_the_reference_interleave():
+    d, ff = 6, 4
+    Wg = torch.arange(d * ff, dtype=torch.float32).reshape(d, ff)
+    Wu = -Wg - 1
+    W13 = fsw_weights.pack_w13(Wg, Wu)
+    assert W13.shape == (2 * ff, d)
+    for j in range(ff):
+        assert torch.equal(W13[2 * j], Wu[:, j])       # even row = up (linear) operand
+        assert torch.equal(W13[2 * j + 1], Wg[:, j])   # odd row = gate (SiLU) operand
+    g2, u2 = fsw_weights.unpack_w13(W13)
+    assert torch.equal(g2, Wg) and torch.equal(u2, Wu)
+    Wd = torch.randn(ff, d)
+    W2 = fsw_weights.pack_wd(Wd)
+    assert W2.shape == (d, ff) and W2.is_contiguous() and torch.equal(W2.T, Wd)
+    # the packed layout evaluates to the unpacked formulation (numeric_tests.py:41-43)
+    X = torch.randn(3, d)
+    C = X @ W13.T
+    H = C[:, 0::2] * torch.nn.functional.silu(C[:, 1::2])
+    assert torch.allclose(H, torch.nn.functional.silu(X @ Wg) * (X @ Wu), atol=1e-5)
+
+
+def test_work_formulas_match_the_published_tables():
+    # FLOPs and bytes of the five configurations
+    want = {"C1": (8858370048, 25165824), "C2": (1108101562368, 517996544), "C3": (2886218022912, 956301312),
+            "C4": (5637144576, 353501184), "C5": (2886218022912, 1711276032)}
+    for name, M, d, ff, dtype, seed, xs in fsw_weights.CONFIGS:
+        assert (fsw_weights.flops(M, d, ff), fsw_weights.hbm_bytes(M, d, ff)) == want[name]
+    assert fsw_weights.reference_gateup_flops(8192, 28672, 4096) == 1924615110656  # bench_swiglu.py:117
+
+
+def test_seeded_inputs_are_reproducible_and_scaled():
+    a = fsw_weights.make_inputs(64, 256, 512, torch.bfloat16, seed=3)
+    b = fsw_weights.make_inputs(64, 256, 512, torch.bfloat16, seed=3)
+    for k in ("X", "W13", "W2"):
+        assert torch.equal(a[k], b[k])
+    assert abs(a["X"].float().std().item() - 1.0) < 0.05
+    assert abs(a["Wg"].float().std().item() * 16 - 1.0) < 0.05          # 1/sqrt(256)
+    assert abs(a["Wd"].float().std().item() * 512 ** 0.5 - 1.0) < 0.05  # 1/sqrt(512)
+
+
+def test_operator_surface_matches_the_reference(ext):
+    # pybind functions (torch_bindings.cpp:31-36)
+    assert callable(ext.fused_swiglu_bf16) and callable(ext.swiglu_fwd_bf16)
+    # dispatcher schemas (torch_bindings.cpp:38-43), byte for byte
+    s1 = str(torch.ops.ASMLLM.fused_swiglu_bf16.default._schema)
+    s2 = str(torch.ops.ASMLLM.swiglu_fwd_bf16.default._schema)
+    assert s1 == "ASMLLM::fused_swiglu_bf16(Tensor X, Tensor W1W3) -> Tensor"
+    assert s2 == ("ASMLLM::swiglu_fwd_bf16(int m, int n, int k, Tensor A, int ldA, Tensor B, int ldB, Tensor C, "
+                  "int ldC) -> ()")
+    for extra in ("fused_swiglu_fp16", "swiglu_down_bf16", "swiglu_down_fp16", "fused_swiglu_mlp_bf16",
+                  "fused_swiglu_mlp_fp16"):
+        assert hasattr(ext, extra) and hasattr(torch.ops.ASMLLM, extra)
+
+
+def test_wrong_dtype_raises_runtime_error_like_the_reference(ext):
+    # swiglu.cu:475-480: TORCH_CHECK on the dtypes -> RuntimeError; fp16/fp32 inputs are rejected by the bf16 op
+    X32, W32 = torch.zeros(4, 8), torch.zeros(6, 8)
+    with pytest.raises(RuntimeError, match="Expected tensor A to be of type"):
+        ext.fused_swiglu_bf16(X32, W32)
+    with pytest.raises(RuntimeError, match="Expected tensor A to be of type"):
+        ext.fused_swiglu_bf16(X32.half(), W32.half())
+    with pytest.raises(RuntimeError, match="Expected tensor B to be of type"):
+        ext.swiglu_fwd_bf16(4, 6, 8, X32.bfloat16(), 8, W32, 8, torch.zeros(4, 6, dtype=torch.bfloat16), 6)
+    with pytest.raises(RuntimeError, match="Expected tensor C to be of type"):
+        ext.swiglu_fwd_bf16(4, 6, 8, X32.bfloat16(), 8, W32.bfloat16(), 8, torch.zeros(4, 6), 6)
+    # CPU tensors of the right dtype are refused (no CPU fallback exists)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ext.fused_swiglu_bf16(X32.bfloat16(), W32.bfloat16())
+    with pytest.raises(RuntimeError):
+        ext.fused_swiglu_bf16(torch.zeros(4, 8, dtype=torch.bfloat16), torch.zeros(6, 16, dtype=torch.bfloat16))

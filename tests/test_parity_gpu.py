@@ -1,0 +1,282 @@
+"""Parity of the HIP path against the CPU oracle on the same seeded inputs, through the C ABI (fsw_capi) and
+through the PyTorch operator surface. Gates: max|d| <= 2e-2 and mean-relative error <= 5e-3 against the fp32/fp64
+formulation (silu(X@Wg) * (X@Wu)) @ Wd; kernel-level checks are tighter (one rounding of a correctly
+accumulated value)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+import fsw_weights
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DEV = "cuda:0"
+
+
+def ulp_rel(dtype):
+    return 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11  # half an ulp, relative
+
+
+def assert_one_rounding(out, ref64, dtype, what, slack=1e-3):
+    """out must be ref rounded once to `dtype`, up to fp32 accumulation-order noise."""
+    out64 = out.detach().cpu().double()
+    err = (out64 - ref64).abs()
+    bound = ref64.abs() * (2 * ulp_rel(dtype)) + slack
+    bad = err > bound
+    assert not bad.any(), "%s: %d elements beyond one rounding; worst |d|=%g at ref=%g" % (
+        what, int(bad.sum()), err[bad].max().item(), ref64[bad][err[bad].argmax()].item())
+
+
+def to_dev(inp):
+    return {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in inp.items()}
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# golden fixtures and small seeded shapes, every kernel variant
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["tiny_bf16", "ragged_fp16", "block_bf16"])
+def test_golden_fixtures(capi, name):
+    z = np.load(os.path.join(GOLDEN, name + ".npz"))
+    tdtype = torch.bfloat16 if int(z["dtype"]) == 0 else torch.float16
+    as_t = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(tdtype).to(DEV)
+    X, W13, W2 = as_t(z["X"]), as_t(z["W13"]), as_t(z["W2"])
+    H = capi.gateup(X, W13)
+    assert_one_rounding(H, torch.from_numpy(z["H"]), tdtype, name + " H")
+    Y = capi.mlp(X, W13, W2)
+    oracle.assert_parity(Y, torch.from_numpy(z["Y"]), name + " Y")
+
+
+SMALL_SHAPES = [  # (M, d, ff): ragged in every dimension, K tails, single rows, tile edges
+    (1, 8, 1), (1, 64, 4), (3, 24, 5), (16, 64, 16), (17, 72, 33), (31, 136, 130), (33, 200, 127),
+    (64, 64, 128), (65, 264, 129), (127, 320, 257), (128, 512, 64), (129, 1000, 131), (255, 128, 255),
+    (256, 256, 256), (257, 64, 300), (300, 448, 520), (513, 96, 260),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", SMALL_SHAPES)
+def test_small_shapes_auto_dispatch(capi, shape, dtype):
+    M, d, ff = shape
+    inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=1000 + M + d + ff, x_scale=0.5 if dtype == torch.float16 else 1.0)
+    g = to_dev(inp)
+    H = capi.gateup(g["X"], g["W13"])
+    H64 = oracle.ref_gateup(inp["X"], inp["W13"], torch.float64)
+    assert_one_rounding(H, H64, dtype, "H %s" % (shape,))
+    # the down kernel on its own: oracle fed with the GPU's H
+    Y = capi.down(H, g["W2"])
+    assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype, "Y|H %s" % (shape,))
+    # whole forward against the unrounded formulation in its unpacked form
+    Yf = capi.mlp(g["X"], g["W13"], g["W2"])
+    assert torch.equal(Yf, Y)
+    oracle.assert_parity(Yf, oracle.ref_mlp_unpacked(inp["X"], inp["Wg"], inp["Wu"], inp["Wd"], torch.float64),
+                         "mlp %s" % (shape,))
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_every_tiled_variant(capi, variant, dtype):
+    try:
+        capi.set_variant(0, variant)
+        capi.set_variant(1, variant)
+        for (M, d, ff) in [(5, 40, 9), (70, 136, 150), (300, 264, 330), (520, 64, 260)]:
+            inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=7 * variant + M, x_scale=0.5)
+            g = to_dev(inp)
+            H = capi.gateup(g["X"], g["W13"])
+            assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype,
+                                "variant %d H %s" % (variant, (M, d, ff)))
+            Y = capi.down(H, g["W2"])
+            assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype,
+                                "variant %d Y %s" % (variant, (M, d, ff)))
+    finally:
+        capi.set_variant(0, -1)
+        capi.set_variant(1, -1)
+
+
+def test_empty_and_degenerate_problems(capi):
+    bf = torch.bfloat16
+    X = torch.randn(0, 64, device=DEV).to(bf)
+    W13 = torch.randn(16, 64, device=DEV).to(bf)
+    W2 = torch.randn(64, 8, device=DEV).to(bf)
+    assert capi.gateup(X, W13).shape == (0, 8)
+    assert capi.mlp(X, W13, W2).shape == (0, 64)
+    # ff = 0: Y = 0
+    X1 = torch.randn(4, 64, device=DEV).to(bf)
+    Y = capi.mlp(X1, torch.empty(0, 64, device=DEV, dtype=bf), torch.empty(64, 0, device=DEV, dtype=bf),
+                 out=torch.full((4, 64), 7.0, device=DEV, dtype=bf))
+    assert Y.abs().max().item() == 0.0
+    # K = 0: up = gate = 0, H = 0 * silu(0) = 0
+    H = capi.gateup(torch.empty(4, 0, device=DEV, dtype=bf), torch.empty(16, 0, device=DEV, dtype=bf),
+                    out=torch.full((4, 8), 7.0, device=DEV, dtype=bf))
+    assert H.abs().max().item() == 0.0
+
+
+def test_even_odd_convention_on_device(capi):
+    """One-hot probe through the HIP kernel: H[m,j] = W13[2j,m] * silu(W13[2j+1,m]) for X = I."""
+    K, ff = 64, 40
+    X = torch.eye(K, dtype=torch.bfloat16, device=DEV)
+    g = torch.Generator().manual_seed(12)
+    W13 = (torch.randn((2 * ff, K), generator=g) * 2).to(torch.bfloat16)
+    H = capi.gateup(X, W13.to(DEV)).cpu()
+    up, gate = W13[0::2].double().T, W13[1::2].double().T
+    assert_one_rounding(H, up * torch.nn.functional.silu(gate), torch.bfloat16, "one-hot", slack=1e-6)
+    swapped = gate * torch.nn.functional.silu(up)
+    assert (H.double() - swapped).abs().max().item() > 0.5
+
+
+def test_exact_small_integer_products_round_once(capi):
+    """K <= 32 and small-integer inputs make every fp32 partial sum exact, so the output must equal the
+    round-to-nearest-even of the exact value bit for bit (no accumulation-order slack)."""
+    for dtype in (torch.bfloat16, torch.float16):
+        g = torch.Generator().manual_seed(21)
+        X = torch.randint(-3, 4, (37, 32), generator=g).to(dtype)
+        W2 = torch.randint(-3, 4, (50, 32), generator=g).to(dtype)
+        Y = capi.down(X.to(DEV), W2.to(DEV)).cpu()
+        exact = X.double() @ W2.double().T
+        assert torch.equal(Y.double(), exact)  # |values| <= 288: exactly representable in both types
+        # ties and inexact values: scale by 1/256 + offsets so many products need rounding
+        Xs = (X.double() * 1.01).to(dtype)
+        Ws = (W2.double() * 0.37).to(dtype)
+        Yr = capi.down(Xs.to(DEV), Ws.to(DEV)).cpu()
+        want = (Xs.double() @ Ws.double().T)
+        want_f32 = want.float()  # K=32 products of 8/11-bit significands: fp32 sums are exact or within 1 fp32 ulp
+        ok = (Yr == want_f32.to(dtype))
+        assert ok.float().mean().item() > 0.995, ok.float().mean().item()
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# operator surface (PyTorch extension), the ldC/2 rule, error behaviour
+# ---------------------------------------------------------------------------------------------------------------
+def test_torch_ops_match_c_abi_and_reference_formulation(capi, ext):
+    inp = fsw_weights.make_inputs(200, 256, 328, torch.bfloat16, seed=33)
+    g = to_dev(inp)
+    H_c = capi.gateup(g["X"], g["W13"])
+    H_p = ext.fused_swiglu_bf16(g["X"], g["W13"])
+    H_o = torch.ops.ASMLLM.fused_swiglu_bf16(g["X"], g["W13"])
+    assert H_p.dtype == torch.bfloat16 and H_p.shape == (200, 328) and H_p.device == g["X"].device
+    assert torch.equal(H_c, H_p) and torch.equal(H_c, H_o)
+    # the reference's own check (numeric_tests.py:41-52): bf16 torch formulation on the GPU
+    C = g["X"] @ g["W13"].T
+    gated = C[:, ::2] * torch.nn.functional.silu(C[:, 1::2])
+    diff = (H_p - gated).float()
+    assert diff.abs().max().item() < 0.1 and (diff.norm() / gated.float().norm()).item() < 2e-2
+    Y = ext.fused_swiglu_mlp_bf16(g["X"], g["W13"], g["W2"])
+    assert torch.equal(Y, capi.mlp(g["X"], g["W13"], g["W2"]))
+    assert torch.equal(Y, torch.ops.ASMLLM.swiglu_down_bf16(H_p, g["W2"]))
+    oracle.assert_parity(Y, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"]), "ext mlp")
+    # fp16 additions
+    i16 = fsw_weights.make_inputs(96, 128, 200, torch.float16, seed=34, x_scale=0.5)
+    g16 = to_dev(i16)
+    Y16 = ext.fused_swiglu_mlp_fp16(g16["X"], g16["W13"], g16["W2"])
+    oracle.assert_parity(Y16, oracle.ref_mlp(i16["X"], i16["W13"], i16["W2"]), "ext mlp fp16")
+    with pytest.raises(RuntimeError):
+        ext.fused_swiglu_bf16(g16["X"], g16["W13"])  # fp16 into the bf16 op (swiglu.cu:475-480)
+
+
+def test_swiglu_fwd_bf16_writes_dense_half_width_rows(ext):
+    """bench_swiglu.py:91,106 passes C as [M, N] with ldC = N; the op writes a dense [M, N/2] matrix with row
+    stride ldC/2 into its first M*N/2 elements (swiglu.cu:353,408,414) and leaves the rest untouched."""
+    M, K, ff = 70, 128, 90
+    N = 2 * ff
+    inp = fsw_weights.make_inputs(M, K, ff, torch.bfloat16, seed=35)
+    g = to_dev(inp)
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert ext.swiglu_fwd_bf16(M, N, K, g["X"], K, g["W13"], K, C, N) is None
+    flat = C.flatten()
+    H = flat[: M * ff].view(M, ff)
+    assert torch.equal(H, ext.fused_swiglu_bf16(g["X"], g["W13"]))
+    assert torch.isnan(flat[M * ff:]).all()
+    # same through the dispatcher, with padded leading dimensions on the inputs
+    Xp = torch.zeros((M, K + 16), dtype=torch.bfloat16, device=DEV)
+    Xp[:, :K] = g["X"]
+    Wp = torch.zeros((N, K + 8), dtype=torch.bfloat16, device=DEV)
+    Wp[:, :K] = g["W13"]
+    C2 = torch.full((M, N + 20), float("nan"), dtype=torch.bfloat16, device=DEV)
+    torch.ops.ASMLLM.swiglu_fwd_bf16(M, N, K, Xp, K + 16, Wp, K + 8, C2, N + 20)
+    H2 = C2.flatten()[: M * (ff + 10)].view(M, ff + 10)
+    assert torch.equal(H2[:, :ff], H) and torch.isnan(H2[:, ff:]).all()
+    with pytest.raises(RuntimeError):
+        ext.swiglu_fwd_bf16(M, N, K, g["X"], K, g["W13"], K, torch.empty(4, 4, dtype=torch.bfloat16, device=DEV), N)
+    with pytest.raises(RuntimeError):
+        ext.swiglu_fwd_bf16(M, N + 1, K, g["X"], K, g["W13"], K, C, N)  # odd N
+
+
+def test_strided_views_and_row_independence(capi):
+    inp = fsw_weights.make_inputs(150, 192, 140, torch.bfloat16, seed=36)
+    g = to_dev(inp)
+    Y = capi.mlp(g["X"], g["W13"], g["W2"])
+    # row m of Y depends on row m of X only: any row subset gives the same rows, bit for bit
+    for rows in (slice(0, 1), slice(17, 18), slice(100, 150), slice(3, 70)):
+        assert torch.equal(capi.mlp(g["X"][rows], g["W13"], g["W2"]), Y[rows])
+    # every second row through a strided view (ldx = 2 * K)
+    assert torch.equal(capi.mlp(g["X"][::2], g["W13"], g["W2"]), Y[::2])
+    # padding with zero rows/features does not change the live part
+    W13z = torch.cat([g["W13"], torch.zeros(24, 192, dtype=torch.bfloat16, device=DEV)])
+    W2z = torch.cat([g["W2"], torch.zeros(192, 12, dtype=torch.bfloat16, device=DEV)], dim=1).contiguous()
+    assert torch.equal(capi.mlp(g["X"], W13z, W2z), Y)
+
+
+def test_permutation_and_linearity_properties(capi):
+    inp = fsw_weights.make_inputs(90, 128, 96, torch.bfloat16, seed=37)
+    g = to_dev(inp)
+    H = capi.gateup(g["X"], g["W13"])
+    perm = torch.randperm(96, generator=torch.Generator().manual_seed(2)).to(DEV)
+    W13p = g["W13"].view(96, 2, 128)[perm].reshape(192, 128).contiguous()
+    assert torch.equal(capi.gateup(g["X"], W13p), H[:, perm])  # features are independent of their position
+    W13u = g["W13"].clone()
+    W13u[0::2] *= 2  # exact in bf16: doubles every H bit-exactly
+    assert torch.equal(capi.gateup(g["X"], W13u).float(), 2 * H.float())
+    Y = capi.down(H, g["W2"])
+    assert torch.equal(capi.down(H, (g["W2"] * 4).contiguous()).float(), 4 * Y.float())
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# the five benchmark configurations at full size
+# ---------------------------------------------------------------------------------------------------------------
+def _config_case(capi, name, sample_rows):
+    inp = fsw_weights.make_config(name)
+    g = {k: inp[k].to(DEV) for k in ("X", "W13", "W2")}
+    M, dtype = inp["M"], inp["dtype"]
+    H = capi.gateup(g["X"], g["W13"])
+    Y = capi.mlp(g["X"], g["W13"], g["W2"])
+    torch.cuda.synchronize()
+    assert torch.isfinite(Y.float()).all()
+    gen = torch.Generator().manual_seed(99)
+    rows = torch.sort(torch.randperm(M, generator=gen)[: min(M, sample_rows)]).values
+    Xs = inp["X"][rows]
+    Href = oracle.ref_gateup(Xs, inp["W13"])
+    Yref = oracle.ref_down(Href, inp["W2"])
+    mh = oracle.assert_parity(H[rows.to(DEV)], Href, name + " H")
+    my = oracle.assert_parity(Y[rows.to(DEV)], Yref, name + " Y")
+    print("\n%s rows=%d H %s\n%s rows=%d Y %s" % (name, len(rows), mh, name, len(rows), my))
+    # size-independent property on the FULL output: Y is linear in W2, so sum_n Y[m, n] = H[m, :] . colsum(W2),
+    # evaluated in fp64 from the GPU's own H for every row
+    colsum = inp["W2"].double().sum(dim=0)
+    want = H.cpu().double() @ colsum
+    got = Y.cpu().double().sum(dim=1)
+    scale = (H.cpu().double().abs() @ inp["W2"].double().abs().sum(dim=0)).clamp_min(1e-6)
+    assert ((got - want).abs() / scale).max().item() < 2e-3
+    return inp, g, H, Y
+
+
+def test_config_c1(capi):
+    inp, g, H, Y = _config_case(capi, "C1", 512)
+    oracle.assert_parity(Y, oracle.ref_mlp_unpacked(inp["X"], inp["Wg"], inp["Wu"], inp["Wd"]), "C1 unpacked")
+
+
+def test_config_c4_decode(capi):
+    _config_case(capi, "C4", 16)
+
+
+def test_config_c2(capi):
+    _config_case(capi, "C2", 192)
+
+
+def test_config_c3_headline(capi):
+    _config_case(capi, "C3", 192)
+
+
+def test_config_c5_fp16(capi):
+    _config_case(capi, "C5", 96)
