@@ -80,7 +80,10 @@ def _stream(t):
 
 
 def _ld(t):
-    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+    """Row stride in elements; degenerate shapes (one row, empty rows) report the row length."""
+    if t.shape[0] > 1 and t.shape[1] > 0:
+        return t.stride(0)
+    return t.shape[1]
 
 
 def gateup(X, W13, out=None):

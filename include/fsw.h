@@ -54,7 +54,8 @@ extern "C" {
  * Host-only argument validation of fsw_gateup (replaces the dtype TORCH_CHECKs of swiglu.cu:475-480 and adds
  * the shape/stride checks the reference leaves out). Rules: M >= 0; N >= 0 and even; K >= 0 and K % 8 == 0
  * (16-byte vectors; the reference needs K % 32 == 0, swiglu.cu:220-230); ldx >= K, ldw >= K, ldh >= N/2;
- * ldx % 8 == 0 and ldw % 8 == 0; pointers non-NULL and X, W13 16-byte aligned when the problem is non-empty.
+ * ldx % 8 == 0 and ldw % 8 == 0; pointers non-NULL and X, W13 16-byte aligned when the problem is non-empty
+ * (M == 0 or N == 0 needs no pointers; K == 0 needs only H, which is then written with zeros).
  */
 FSW_API int fsw_validate_gateup(int dtype, int64_t M, int64_t N, int64_t K,
                         const void* X, int64_t ldx, const void* W13, int64_t ldw,

@@ -18,9 +18,9 @@ import fsw_weights  # noqa: E402
 
 # name, M, d, ff, dtype, seed, x_scale
 CASES = [
-    ("tiny_bf16", 5, 16, 6, torch.bfloat16, 101, 1.0),
+    ("tiny_bf16", 5, 16, 8, torch.bfloat16, 101, 1.0),
     ("ragged_fp16", 17, 40, 12, torch.float16, 102, 0.5),
-    ("block_bf16", 24, 64, 36, torch.bfloat16, 103, 1.0),
+    ("block_bf16", 24, 64, 40, torch.bfloat16, 103, 1.0),
 ]
 
 

@@ -45,14 +45,23 @@ def test_golden_fixtures(capi, name):
     X, W13, W2 = as_t(z["X"]), as_t(z["W13"]), as_t(z["W2"])
     H = capi.gateup(X, W13)
     assert_one_rounding(H, torch.from_numpy(z["H"]), tdtype, name + " H")
+    if H.shape[1] % 8:
+        # the down projection reads H and W2 in 16-byte vectors along ff: ff % 8 != 0 is refused, not mis-computed
+        with pytest.raises(capi.FswError) as ei:
+            capi.mlp(X, W13, W2)
+        assert ei.value.code == capi.E_ALIGN
+        return
     Y = capi.mlp(X, W13, W2)
     oracle.assert_parity(Y, torch.from_numpy(z["Y"]), name + " Y")
 
 
-SMALL_SHAPES = [  # (M, d, ff): ragged in every dimension, K tails, single rows, tile edges
-    (1, 8, 1), (1, 64, 4), (3, 24, 5), (16, 64, 16), (17, 72, 33), (31, 136, 130), (33, 200, 127),
-    (64, 64, 128), (65, 264, 129), (127, 320, 257), (128, 512, 64), (129, 1000, 131), (255, 128, 255),
-    (256, 256, 256), (257, 64, 300), (300, 448, 520), (513, 96, 260),
+SMALL_SHAPES = [  # (M, d, ff) with ff % 8 == 0: ragged M and d, K tails, single rows, tile edges
+    (1, 8, 8), (1, 64, 8), (3, 24, 16), (16, 64, 16), (17, 72, 40), (31, 136, 136), (33, 200, 120),
+    (64, 64, 128), (65, 264, 136), (127, 320, 264), (128, 512, 64), (129, 1000, 136), (255, 128, 248),
+    (256, 256, 256), (257, 64, 304), (300, 448, 520), (513, 96, 264),
+]
+GATEUP_ONLY_SHAPES = [  # any ff (odd, prime, below one vector): exercises the scalar store path and odd ldh
+    (1, 8, 1), (3, 24, 5), (17, 72, 33), (33, 200, 127), (65, 264, 129), (129, 64, 131), (255, 128, 255), (70, 32, 3),
 ]
 
 
@@ -75,13 +84,22 @@ def test_small_shapes_auto_dispatch(capi, shape, dtype):
                          "mlp %s" % (shape,))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", GATEUP_ONLY_SHAPES)
+def test_gateup_any_ff(capi, shape, dtype):
+    M, d, ff = shape
+    inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=2000 + M + d + ff, x_scale=0.5)
+    H = capi.gateup(inp["X"].to(DEV), inp["W13"].to(DEV))
+    assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "H %s" % (shape,))
+
+
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_every_tiled_variant(capi, variant, dtype):
     try:
         capi.set_variant(0, variant)
         capi.set_variant(1, variant)
-        for (M, d, ff) in [(5, 40, 9), (70, 136, 150), (300, 264, 330), (520, 64, 260)]:
+        for (M, d, ff) in [(5, 40, 8), (70, 136, 152), (300, 264, 328), (520, 64, 264)]:
             inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=7 * variant + M, x_scale=0.5)
             g = to_dev(inp)
             H = capi.gateup(g["X"], g["W13"])
@@ -115,7 +133,7 @@ def test_empty_and_degenerate_problems(capi):
 
 def test_even_odd_convention_on_device(capi):
     """One-hot probe through the HIP kernel: H[m,j] = W13[2j,m] * silu(W13[2j+1,m]) for X = I."""
-    K, ff = 64, 40
+    K, ff = 64, 41
     X = torch.eye(K, dtype=torch.bfloat16, device=DEV)
     g = torch.Generator().manual_seed(12)
     W13 = (torch.randn((2 * ff, K), generator=g) * 2).to(torch.bfloat16)
@@ -204,7 +222,7 @@ def test_swiglu_fwd_bf16_writes_dense_half_width_rows(ext):
 
 
 def test_strided_views_and_row_independence(capi):
-    inp = fsw_weights.make_inputs(150, 192, 140, torch.bfloat16, seed=36)
+    inp = fsw_weights.make_inputs(150, 192, 144, torch.bfloat16, seed=36)
     g = to_dev(inp)
     Y = capi.mlp(g["X"], g["W13"], g["W2"])
     # row m of Y depends on row m of X only: any row subset gives the same rows, bit for bit
@@ -213,8 +231,8 @@ def test_strided_views_and_row_independence(capi):
     # every second row through a strided view (ldx = 2 * K)
     assert torch.equal(capi.mlp(g["X"][::2], g["W13"], g["W2"]), Y[::2])
     # padding with zero rows/features does not change the live part
-    W13z = torch.cat([g["W13"], torch.zeros(24, 192, dtype=torch.bfloat16, device=DEV)])
-    W2z = torch.cat([g["W2"], torch.zeros(192, 12, dtype=torch.bfloat16, device=DEV)], dim=1).contiguous()
+    W13z = torch.cat([g["W13"], torch.zeros(32, 192, dtype=torch.bfloat16, device=DEV)])
+    W2z = torch.cat([g["W2"], torch.zeros(192, 16, dtype=torch.bfloat16, device=DEV)], dim=1).contiguous()
     assert torch.equal(capi.mlp(g["X"], W13z, W2z), Y)
 
 
@@ -248,7 +266,10 @@ def _config_case(capi, name, sample_rows):
     Xs = inp["X"][rows]
     Href = oracle.ref_gateup(Xs, inp["W13"])
     Yref = oracle.ref_down(Href, inp["W2"])
-    mh = oracle.assert_parity(H[rows.to(DEV)], Href, name + " H")
+    # H reaches |H| > 8, where half an ulp of bf16 alone is 0.031: the absolute gate is a statement about the
+    # forward's output Y; H is held to "one rounding of the fp32 value" and to the relative gates instead.
+    assert_one_rounding(H[rows.to(DEV)], Href.double(), dtype, name + " H", slack=2e-3)
+    mh = oracle.assert_parity(H[rows.to(DEV)], Href, name + " H", max_abs_tol=float("inf"))
     my = oracle.assert_parity(Y[rows.to(DEV)], Yref, name + " Y")
     print("\n%s rows=%d H %s\n%s rows=%d Y %s" % (name, len(rows), mh, name, len(rows), my))
     # size-independent property on the FULL output: Y is linear in W2, so sum_n Y[m, n] = H[m, :] . colsum(W2),
