@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X fused SwiGLU MLP forward: one JSON line on stdout.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--no-cpu] [--detail]
+
+A step is one whole forward Y = (silu(X @ Wg) * (X @ Wu)) @ Wd over one batch of seeded synthetic input that is
+already resident in HBM: the gated dual-GEMM kernel followed by the down-projection kernel, both launched
+through the C ABI (libfsw_hip.so) on torch's current stream. `value` is 6*M*d*ff FLOPs per step over the wall
+time of exactly K steps between two device synchronisations. The default workload is the headline configuration
+(Llama-3-8B MLP prefill: M=8192, d=4096, ff=14336, bf16, seed 2).
+
+Extra objects on the same line:
+  roofline     — the gate/up kernel (2/3 of the FLOPs): algorithmic FLOPs / its average duration, measured with
+                 HIP events recorded around that launch inside the timed steps, against the bf16 dense MFMA peak;
+  cpu_baseline — the same formulation in fp32 PyTorch on this host's cores (oracle/, the checker) on a bounded
+                 row sample of the same workload; the rows it computes also serve as a parity spot check;
+  decode       — the M=16 weight-streaming configuration in GB/s against the HBM3E peak.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "fused-swiglu_amd"))
+
+MFMA_PEAK_TFLOPS = 2516.6  # MI355X dense bf16/fp16: 256 CU x 2.4 GHz x 4096 flop/clk/CU
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="C3", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the cpu_baseline sample")
+    ap.add_argument("--detail", action="store_true", help="also time every configuration (stderr table)")
+    return ap.parse_args()
+
+
+def run_steps(capi, torch, g, cfg, steps, warmup, with_events=True):
+    """Times exactly `steps` forwards. Returns (wall seconds, [gate/up ms], [down ms])."""
+    import fsw_capi
+    L = capi.lib()
+    M, d, ff = cfg["M"], cfg["d"], cfg["ff"]
+    code = fsw_capi.dtype_code(g["X"])
+    H = torch.empty((M, ff), dtype=g["X"].dtype, device=g["X"].device)
+    Y = torch.empty((M, d), dtype=g["X"].dtype, device=g["X"].device)
+    ws_bytes = L.fsw_down_workspace_bytes(code, M, d, ff)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=g["X"].device)
+    stream = torch.cuda.current_stream().cuda_stream
+    xp, wp, w2p, hp, yp, wsp = (t.data_ptr() for t in (g["X"], g["W13"], g["W2"], H, Y, ws))
+
+    def step(ev=None):
+        if ev is not None:
+            ev[0].record()
+        rc = L.fsw_gateup(code, M, 2 * ff, d, xp, d, wp, d, hp, ff, stream)
+        if ev is not None:
+            ev[1].record()
+        rc2 = L.fsw_down(code, M, d, ff, hp, ff, w2p, ff, yp, d, wsp, ws_bytes, stream)
+        if ev is not None:
+            ev[2].record()
+        if rc or rc2:
+            raise RuntimeError("fsw launch failed: %s / %s" % (capi.strerror(rc), capi.strerror(rc2)))
+
+    for _ in range(warmup):
+        step()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)] if with_events else None
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(events[i] if events else None)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    gu = [e[0].elapsed_time(e[1]) for e in events] if events else []
+    dn = [e[1].elapsed_time(e[2]) for e in events] if events else []
+    return wall, gu, dn, Y
+
+
+def cpu_baseline(torch, inp, cfg, budget_s, y_gpu):
+    """fp32 PyTorch formulation on the host cores over a row sample of the workload, repeated for ~budget_s."""
+    from oracle import oracle
+    import fsw_weights
+    M, d, ff = cfg["M"], cfg["d"], cfg["ff"]
+    threads = torch.get_num_threads()
+    rows = min(M, 256)
+    gen = torch.Generator().manual_seed(1234)
+    idx = torch.sort(torch.randperm(M, generator=gen)[:rows]).values
+    Xs = inp["X"][idx].float()
+    W13f, W2f = inp["W13"].float(), inp["W2"].float()  # upcast once, outside the timed passes
+    oracle.ref_mlp(Xs[:8], W13f, W2f)  # warm-up
+    passes, t_total, Yref = 0, 0.0, None
+    while passes < 1 or (t_total < budget_s and passes < 200):
+        t0 = time.perf_counter()
+        Yref = oracle.ref_mlp(Xs, W13f, W2f)
+        t_total += time.perf_counter() - t0
+        passes += 1
+    tflops = fsw_weights.flops(rows, d, ff) * passes / t_total / 1e12
+    parity = oracle.error_metrics(y_gpu[idx.to(y_gpu.device)], Yref)
+    parity["rows"] = rows
+    parity["pass"] = bool(oracle.passes(parity))
+    base = {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "%d of %d rows of %s, %d passes of the fp32 torch formulation in %.1f s" % (
+                rows, M, cfg["name"], passes, t_total)}
+    return base, parity
+
+
+def med(xs):
+    s = sorted(xs)
+    return s[len(s) // 2] if s else float("nan")
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards over rows or "
+              "over ff with one all-reduce, which is not part of this build)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    import fsw_capi as capi
+    import fsw_weights
+    capi.lib()
+    torch.cuda.set_device(0)
+
+    def load(name):
+        inp = fsw_weights.make_config(name)
+        g = {k: inp[k].to("cuda:0") for k in ("X", "W13", "W2")}
+        return inp, g
+
+    inp, g = load(args.workload)
+    cfg = {k: inp[k] for k in ("name", "M", "d", "ff", "seed")}
+    M, d, ff = cfg["M"], cfg["d"], cfg["ff"]
+    dtype_name = "bf16" if inp["dtype"] == torch.bfloat16 else "fp16"
+    wall, gu, dn, Y = run_steps(capi, torch, g, cfg, args.steps, args.warmup)
+    ms_per_step = wall / args.steps * 1e3
+    tflops = fsw_weights.flops(M, d, ff) / (ms_per_step * 1e-3) / 1e12
+    gu_ms, dn_ms = sum(gu) / len(gu), sum(dn) / len(dn)
+    gu_tflops = fsw_weights.gateup_flops(M, d, ff) / (gu_ms * 1e-3) / 1e12
+    dn_tflops = 2 * M * d * ff / (dn_ms * 1e-3) / 1e12
+    hbm_bound = args.workload == "C4"
+    if hbm_bound:
+        gu_bytes = (2 * ff * d + M * d + M * ff) * 2
+        roofline = {"bound": "hbm", "kernel": capi.variant_name(0, 0, M, 2 * ff, d) + " (gate/up)",
+                    "achieved": round(gu_bytes / (gu_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(gu_bytes / (gu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                    "avg_kernel_ms": round(gu_ms, 5)}
+    else:
+        roofline = {"bound": "mfma", "kernel": capi.variant_name(0, 0, M, 2 * ff, d) + " (gate/up)",
+                    "achieved": round(gu_tflops, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(gu_tflops / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                    "avg_kernel_ms": round(gu_ms, 5)}
+    out = {
+        "metric": "fused SwiGLU fwd TFLOP/s + % bf16 MFMA peak (M=8192,d=4096,ff=14336)",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype_name, "data": "synthetic",
+        "config": {"workload": "%s: SwiGLU MLP forward M=%d d=%d ff=%d %s seed %d" % (
+            cfg["name"], M, d, ff, dtype_name, cfg["seed"]), "M": M, "d": d, "ff": ff},
+        "frac_of_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS, 4),
+        "kernels": {"gateup_ms": round(gu_ms, 5), "gateup_ms_median": round(med(gu), 5),
+                    "gateup_tflops": round(gu_tflops, 2), "down_ms": round(dn_ms, 5),
+                    "down_tflops": round(dn_tflops, 2),
+                    "hbm_gbs": round(fsw_weights.hbm_bytes(M, d, ff) / (ms_per_step * 1e-3) / 1e9, 2)},
+        "roofline": roofline,
+    }
+
+    # decode leg: M = 16, weight streaming, judged in GB/s
+    if args.workload != "C4":
+        inp4, g4 = load("C4")
+        c4 = {k: inp4[k] for k in ("name", "M", "d", "ff", "seed")}
+        wall4, gu4, dn4, _ = run_steps(capi, torch, g4, c4, 200, 20)
+        ms4 = wall4 / 200 * 1e3
+        by4 = fsw_weights.hbm_bytes(c4["M"], c4["d"], c4["ff"])
+        out["decode"] = {"workload": "C4: M=16 d=4096 ff=14336 bf16 seed 3", "ms_per_step": round(ms4, 5),
+                         "value": round(by4 / (ms4 * 1e-3) / 1e9, 2), "unit": "GB/s", "peak": HBM_PEAK_GBS,
+                         "frac": round(by4 / (ms4 * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                         "gateup_ms": round(sum(gu4) / len(gu4), 5), "down_ms": round(sum(dn4) / len(dn4), 5)}
+        del inp4, g4
+
+    if args.detail:
+        for name in ("C1", "C2", "C3", "C4", "C5"):
+            i2, g2 = load(name)
+            c2 = {k: i2[k] for k in ("name", "M", "d", "ff", "seed")}
+            n = 200 if name in ("C1", "C4") else 30
+            w2, a2, b2, _ = run_steps(capi, torch, g2, c2, n, 5)
+            ms2 = w2 / n * 1e3
+            print("%s  %.4f ms/step  %.1f TFLOP/s  %.1f GB/s  gate/up %.4f ms  down %.4f ms" % (
+                name, ms2, fsw_weights.flops(c2["M"], c2["d"], c2["ff"]) / ms2 / 1e9,
+                fsw_weights.hbm_bytes(c2["M"], c2["d"], c2["ff"]) / ms2 / 1e6, med(a2), med(b2)), file=sys.stderr)
+            del i2, g2
+
+    if not args.no_cpu:
+        base, parity = cpu_baseline(torch, inp, cfg, args.cpu_seconds, Y)
+        out["cpu_baseline"] = base
+        out["parity_spot_check"] = {k: (round(v, 6) if isinstance(v, float) else v) for k, v in parity.items()}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
