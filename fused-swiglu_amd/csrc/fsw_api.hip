@@ -53,7 +53,8 @@ int pick_tiled(int64_t m, int64_t np) {
 
 int resolve_variant(int family, int64_t m, int64_t np) {
   const int forced = g_forced_variant[family];
-  if (forced >= 0) return forced;
+  if (forced >= 0 && !(forced == VARIANT_SKINNY && m > 64)) return forced;
+  if (m <= 16) return VARIANT_SKINNY;  // decode: weight streaming, HBM bound
   return pick_tiled(m, np);
 }
 
@@ -155,7 +156,7 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
   a.nq = (int)M;
   a.k = (int)K;
   const int v = resolve_variant(0, M, N);
-  if (v == VARIANT_SKINNY) return FSW_E_VARIANT;
+  if (v == VARIANT_SKINNY) return finish(fsw::launch_skinny(dtype, true, a, nullptr, (hipStream_t)stream));
   return finish(fsw::launch_tiled(v, dtype, true, a, (hipStream_t)stream));
 }
 
@@ -187,7 +188,7 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
   a.nq = (int)M;
   a.k = (int)FF;
   const int v = resolve_variant(1, M, D);
-  if (v == VARIANT_SKINNY) return FSW_E_VARIANT;
+  if (v == VARIANT_SKINNY) return finish(fsw::launch_skinny(dtype, false, a, workspace, (hipStream_t)stream));
   return finish(fsw::launch_tiled(v, dtype, false, a, (hipStream_t)stream));
 }
 

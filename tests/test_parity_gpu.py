@@ -113,6 +113,32 @@ def test_every_tiled_variant(capi, variant, dtype):
         capi.set_variant(1, -1)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 33, 48, 64])
+def test_skinny_weight_streaming_variant(capi, M, dtype):
+    """The decode kernels (forced for every M <= 64 here; picked automatically for M <= 16)."""
+    try:
+        capi.set_variant(0, 100)
+        capi.set_variant(1, 100)
+        for (d, ff) in [(8, 8), (136, 40), (1000, 264), (4096, 520), (256, 2056)]:
+            inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=31 * M + d, x_scale=0.5)
+            g = to_dev(inp)
+            assert capi.variant_name(0, 0, M, 2 * ff, d) == "skinny"
+            H = capi.gateup(g["X"], g["W13"])
+            assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype,
+                                "skinny H %s" % ((M, d, ff),))
+            Y = capi.down(H, g["W2"])
+            assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype,
+                                "skinny Y %s" % ((M, d, ff),))
+        # odd ff: scalar stores, odd ldh
+        inp = fsw_weights.make_inputs(M, 72, 37, dtype, seed=5, x_scale=0.5)
+        H = capi.gateup(inp["X"].to(DEV), inp["W13"].to(DEV))
+        assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "skinny odd ff")
+    finally:
+        capi.set_variant(0, -1)
+        capi.set_variant(1, -1)
+
+
 def test_empty_and_degenerate_problems(capi):
     bf = torch.bfloat16
     X = torch.randn(0, 64, device=DEV).to(bf)
