@@ -91,6 +91,10 @@ const char* fsw_strerror(int code) {
 int fsw_last_hip_error(void) { return g_last_hip_error; }
 
 int fsw_set_variant(int family, int variant) {
+  if (family == 2) {  // tuning knob: raster band height of the tiled kernels
+    fsw::set_raster_group(variant);
+    return FSW_OK;
+  }
   if (family < 0 || family > 1) return FSW_E_VARIANT;
   if (variant >= 0 && variant != VARIANT_SKINNY && variant >= fsw::tiled_variant_count()) return FSW_E_VARIANT;
   g_forced_variant[family] = variant < 0 ? -1 : variant;

@@ -22,6 +22,50 @@
 
 namespace fsw {
 
+// Epilogue shared by the tiled kernels. A lane owns activation row m = l32 of each Q fragment and, per group
+// of 4 accumulator registers, 4 consecutive output features: feature = 8 * (i / 4) + 4 * hi + (i % 4) within
+// the fragment. Gating (fp32 multiply and SiLU, swiglu.cu:380-381) happens here, then ONE rounding and an
+// 8-byte store.
+template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
+__device__ __forceinline__ void store_tile(f32x16 (&acc)[FP][FQ], const GemmArgs& a, int p0, int q0, int wp, int wq,
+                                           int l32, int hi) {
+  unsigned short* O = (unsigned short*)a.O;
+  const int nout = GATED ? a.np / 2 : a.np;
+  const bool vec_ok = ((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 7) == 0);
+  constexpr int FO = GATED ? FP / 2 : FP;
+#pragma unroll
+  for (int g = 0; g < FQ; ++g) {
+    const int m = q0 + (wq * FQ + g) * 32 + l32;
+    if (m >= a.nq) continue;
+    unsigned short* orow = O + (long long)m * a.ldo;
+#pragma unroll
+    for (int f = 0; f < FO; ++f) {
+      const int nb = (GATED ? p0 / 2 + (wp * FO + f) * 32 : p0 + (wp * FO + f) * 32) + hi * 4;
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (GATED) {
+            v[e] = acc[f][g][i4 * 4 + e] * silu_f32(acc[f + FO][g][i4 * 4 + e]);
+          } else {
+            v[e] = acc[f][g][i4 * 4 + e];
+          }
+        }
+        const int n = nb + i4 * 8;
+        if (vec_ok && n + 3 < nout) {
+          u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
+          *(u32x2*)(orow + n) = pk;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < nout) orow[n + e] = E::cvt1(v[e]);
+        }
+      }
+    }
+  }
+}
+
 template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
 __global__ void __launch_bounds__(WP* WQ * 64)
 tiled_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
@@ -197,43 +241,183 @@ tiled_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int g
     }
   }
 
-  // ---- epilogue: lane owns activation row m = l32 of each Q fragment and, per group of 4 accumulator
-  // registers, 4 consecutive output features: feature = 8 * (i / 4) + 4 * hi + (i % 4) within the fragment.
-  unsigned short* O = (unsigned short*)a.O;
-  const int nout = GATED ? a.np / 2 : a.np;
-  const bool vec_ok = ((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 7) == 0);
-  constexpr int FO = GATED ? FP / 2 : FP;
+  store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
+}
+
+// ---- direct-to-LDS variant ---------------------------------------------------------------------------------
+// Same tiling and epilogue, but the operand tiles go from global memory straight into LDS with
+// buffer_load_dwordx4 ... lds (no staging registers, no ds_write: LDS writes by ds_write_b128 run at roughly a
+// third of the read rate on this chip and were the largest single cost of the register-staged loop).
+// An LDS-DMA instruction writes lane i's 16 bytes at base + 16 i, so a wave instruction fills 8 consecutive
+// 128-byte rows; the swizzle is applied on the global side: the lane that lands on chunk position p of row r
+// fetches logical chunk p ^ ((r >> 1) & 7). With that function any 16 consecutive rows at one logical chunk
+// cover all 64 banks once (the LDS serves ds_read_b128 sixteen lanes per clock), so operand reads are
+// conflict-free. The two stages are separate __shared__ objects so that the compiler's counter tracking can
+// tell reads of the live stage from DMA writes into the other one.
+typedef __attribute__((address_space(3))) void lds_void;
+
+template <class E, bool GATED, bool KTAIL, int WP, int WQ, int FP, int FQ>
+__global__ void __launch_bounds__(WP* WQ * 64)
+tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
+  constexpr int NT = WP * WQ * 64;
+  constexpr int BP = WP * FP * 32;
+  constexpr int BQ = WQ * FQ * 32;
+  constexpr int BK = 64;
+  constexpr int ROWB = BK * 2;
+  constexpr int RSTEP = NT / 8;
+  constexpr int LP = BP / RSTEP;
+  constexpr int LQ = BQ / RSTEP;
+  constexpr int STAGE = (BP + BQ) * ROWB;
+  static_assert(BP % RSTEP == 0 && BQ % RSTEP == 0 && RSTEP % 16 == 0, "copy mapping");
+  static_assert(!GATED || (FP % 2 == 0), "gated kernel pairs fragments");
+  static_assert(2 * STAGE <= 160 * 1024, "LDS budget of a gfx950 CU");
+
+  __shared__ __align__(1024) unsigned char lds0[STAGE];
+  __shared__ __align__(1024) unsigned char lds1[STAGE];
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // wave-uniform: LDS-DMA bases live in SGPRs
+  const int wq = wave % WQ;
+  const int wp = wave / WQ;
+  const int l32 = lane & 31;
+  const int hi = lane >> 5;
+
+  int tp, tq;
+  tile_coords(blockIdx.x, tiles_p, tiles_q, group, tp, tq);
+  const int p0 = tp * BP;
+  const int q0 = tq * BQ;
+
+  // ---- global -> LDS copy mapping: lane lands on chunk position pc of row rb (+ i * RSTEP)
+  const int pc = t & 7;
+  const int rb = t >> 3;
+  const int lc = pc ^ ((rb >> 1) & 7);  // logical chunk this lane fetches (RSTEP % 16 == 0 keeps (row >> 1) & 7)
+  const unsigned char* pbase = (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
+  const unsigned char* qbase = (const unsigned char*)a.Q + (long long)q0 * a.ldq * 2;
+  const __amdgpu_buffer_rsrc_t prs = make_rsrc(pbase, ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
+  const __amdgpu_buffer_rsrc_t qrs = make_rsrc(qbase, ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2);
+  unsigned poff[LP], qoff[LQ];
 #pragma unroll
-  for (int g = 0; g < FQ; ++g) {
-    const int m = q0 + (wq * FQ + g) * 32 + l32;
-    if (m >= a.nq) continue;
-    unsigned short* orow = O + (long long)m * a.ldo;
-#pragma unroll
-    for (int f = 0; f < FO; ++f) {
-      const int nb = (GATED ? p0 / 2 + (wp * FO + f) * 32 : p0 + (wp * FO + f) * 32) + hi * 4;
-#pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (GATED) {
-            v[e] = acc[f][g][i4 * 4 + e] * silu_f32(acc[f + FO][g][i4 * 4 + e]);
-          } else {
-            v[e] = acc[f][g][i4 * 4 + e];
-          }
-        }
-        const int n = nb + i4 * 8;
-        if (vec_ok && n + 3 < nout) {
-          u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
-          *(u32x2*)(orow + n) = pk;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n + e < nout) orow[n + e] = E::cvt1(v[e]);
-        }
-      }
-    }
+  for (int i = 0; i < LP; ++i) {
+    const int r = rb + i * RSTEP;
+    const int grow = GATED ? (r < BP / 2 ? 2 * r : 2 * (r - BP / 2) + 1) : r;
+    poff[i] = (unsigned)grow * (unsigned)a.ldp * 2u + (unsigned)lc * 16u;
   }
+#pragma unroll
+  for (int i = 0; i < LQ; ++i) {
+    const int r = rb + i * RSTEP;
+    qoff[i] = (unsigned)r * (unsigned)a.ldq * 2u + (unsigned)lc * 16u;
+  }
+
+  // ---- LDS -> MFMA fragment read mapping
+  unsigned xo[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) xo[ks] = (unsigned)((((ks << 1) | hi) ^ ((l32 >> 1) & 7)) * 16);
+  const unsigned rd_p = (unsigned)((GATED ? wp * (FP / 2) * 32 : wp * FP * 32) + l32) * ROWB;
+  const unsigned rd_q = (unsigned)(BP + wq * FQ * 32 + l32) * ROWB;
+  auto p_frag_off = [](int f) -> unsigned {
+    if (GATED) return (unsigned)((f < FP / 2 ? f * 32 : BP / 2 + (f - FP / 2) * 32) * ROWB);
+    return (unsigned)(f * 32 * ROWB);
+  };
+
+  f32x16 acc[FP][FQ];
+#pragma unroll
+  for (int f = 0; f < FP; ++f)
+#pragma unroll
+    for (int g = 0; g < FQ; ++g)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[f][g][i] = 0.0f;
+
+  const int nkt = (a.k + BK - 1) / BK;
+
+  // DMA of K tile `kt` into `stage`: wave-uniform LDS base per instruction, loop-invariant per-lane offset in a
+  // VGPR, the K offset in an SGPR. Rows beyond the matrix are out of range for the buffer descriptor and arrive
+  // as zeros. A prefetch past the last tile re-reads the last tile (never consumed). Only when K is not a
+  // multiple of 64 (KTAIL) do lanes whose chunk lies at or beyond K redirect their offset out of range.
+  auto dma = [&](unsigned char* stage, int kt) {
+    const int ktc = kt < nkt ? kt : nkt - 1;
+    const int kb = ktc * (BK * 2);
+    const bool in = !KTAIL || (ktc * BK + lc * 8) < a.k;
+#pragma unroll
+    for (int i = 0; i < LP; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(stage + i * RSTEP * ROWB + wave * 1024), 16,
+                                               (int)(in ? poff[i] : OOB_OFFSET), kb, 0, 0);
+#pragma unroll
+    for (int i = 0; i < LQ; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(stage + (BP + i * RSTEP) * ROWB + wave * 1024), 16,
+                                               (int)(in ? qoff[i] : OOB_OFFSET), kb, 0, 0);
+  };
+
+  u32x4 pf[2][FP], qf[2][FQ];
+  auto f_read = [&](int fb, const unsigned char* base, int ks) {
+    pf[fb][0] = *(const u32x4*)(base + rd_p + p_frag_off(0) + xo[ks]);
+#pragma unroll
+    for (int g = 0; g < FQ; ++g) qf[fb][g] = *(const u32x4*)(base + rd_q + g * 32 * ROWB + xo[ks]);
+#pragma unroll
+    for (int f = 1; f < FP; ++f) pf[fb][f] = *(const u32x4*)(base + rd_p + p_frag_off(f) + xo[ks]);
+  };
+  auto mma = [&](int fb, int f_lo, int f_hi) {
+#pragma unroll
+    for (int f = f_lo; f < f_hi; ++f)
+#pragma unroll
+      for (int g = 0; g < FQ; ++g) acc[f][g] = E::mfma32(pf[fb][f], qf[fb][g], acc[f][g]);
+  };
+
+  constexpr int NM = FP * FQ;
+  constexpr int NR = FP + FQ;
+  constexpr int NL = LP + LQ;
+  constexpr int HF = FP / 2 > 0 ? FP / 2 : 1;
+  constexpr int MPR = NM / NR > 0 ? NM / NR : 1;
+
+  // One K tile. On entry: stage `cur` holds tile kt (made visible by the previous barrier) and its step-0
+  // fragments are in pf[0]/qf[0]; every wave is done reading `oth`. The DMA of tile kt+1 into `oth` is issued
+  // in step 0 and has the whole iteration to land before the barrier in step 3.
+  auto iteration = [&](unsigned char* cur, unsigned char* oth, int kt) {
+    dma(oth, kt + 1);
+    f_read(1, cur, 1);
+    mma(0, 0, FP);
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);
+      __builtin_amdgcn_sched_group_barrier(0x010, (NL + NR - 1) / NR, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    f_read(0, cur, 2);
+    mma(1, 0, FP);
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    f_read(1, cur, 3);
+    mma(0, 0, FP);
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    mma(1, 0, HF);
+    __syncthreads();  // waits for this wave's DMA (vmcnt) and LDS reads, then for every other wave
+    f_read(0, oth, 0);
+    mma(1, HF, FP);
+#pragma unroll
+    for (int i = 0; i < (FP - HF) * FQ; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x100, (NR + (FP - HF) * FQ - 1) / ((FP - HF) * FQ), 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+  };
+
+  if (nkt > 0) dma(lds0, 0);
+  __syncthreads();
+  if (nkt > 0) f_read(0, lds0, 0);
+  int kt = 0;
+  for (; kt + 1 < nkt; kt += 2) {
+    iteration(lds0, lds1, kt);
+    iteration(lds1, lds0, kt + 1);
+  }
+  if (kt < nkt) iteration(lds0, lds1, kt);
+
+  store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
 }
 
 // ---- variant table ------------------------------------------------------------------------------------
@@ -245,7 +429,12 @@ const TiledVariant kVariants[] = {
     {"tiled_128x128", 128, 128, 256},
     {"tiled_256x64", 256, 64, 256},
     {"tiled_256x32", 256, 32, 256},
+    {"dma_256x256", 256, 256, 256},    // direct-to-LDS copies, conflict-free operand reads
+    {"dma_256x128", 256, 128, 256},
+    {"dma_128x128", 128, 128, 256},
 };
+
+int g_raster_group = 4;
 
 template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
 hipError_t launch_one(const GemmArgs& a, hipStream_t stream) {
@@ -253,9 +442,24 @@ hipError_t launch_one(const GemmArgs& a, hipStream_t stream) {
   const int tiles_p = (a.np + BP - 1) / BP;
   const int tiles_q = (a.nq + BQ - 1) / BQ;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
-  const int group = 4;
   hipLaunchKernelGGL((tiled_kernel<E, GATED, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)), dim3(WP * WQ * 64), 0,
-                     stream, a, tiles_p, tiles_q, group);
+                     stream, a, tiles_p, tiles_q, g_raster_group);
+  return hipGetLastError();
+}
+
+template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
+hipError_t launch_dma(const GemmArgs& a, hipStream_t stream) {
+  constexpr int BP = WP * FP * 32, BQ = WQ * FQ * 32;
+  const int tiles_p = (a.np + BP - 1) / BP;
+  const int tiles_q = (a.nq + BQ - 1) / BQ;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  if (a.k % 64 == 0) {
+    hipLaunchKernelGGL((tiled_dma_kernel<E, GATED, false, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
+                       dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, g_raster_group);
+  } else {
+    hipLaunchKernelGGL((tiled_dma_kernel<E, GATED, true, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
+                       dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, g_raster_group);
+  }
   return hipGetLastError();
 }
 
@@ -267,12 +471,16 @@ hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
     case 2: return launch_one<E, GATED, 2, 2, 2, 2>(a, stream);
     case 3: return launch_one<E, GATED, 4, 1, 2, 2>(a, stream);
     case 4: return launch_one<E, GATED, 4, 1, 2, 1>(a, stream);
+    case 5: return launch_dma<E, GATED, 2, 2, 4, 4>(a, stream);
+    case 6: return launch_dma<E, GATED, 2, 2, 4, 2>(a, stream);
+    case 7: return launch_dma<E, GATED, 2, 2, 2, 2>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
 }  // namespace
 
+void set_raster_group(int g) { g_raster_group = g > 0 ? g : 4; }
 int tiled_variant_count() { return (int)(sizeof(kVariants) / sizeof(kVariants[0])); }
 const TiledVariant& tiled_variant(int variant) { return kVariants[variant]; }
 
