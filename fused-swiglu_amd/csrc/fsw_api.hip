@@ -42,20 +42,21 @@ int check_device() {
 
 // Variant choice for the tiled kernels: the widest tile whose activation-row extent is not mostly padding,
 // stepping down to 128x128 when a 256-wide grid would leave most of the 256 CUs idle.
-int pick_tiled(int64_t m, int64_t np) {
-  if (m <= 32) return 4;   // 256 x 32
-  if (m <= 64) return 3;   // 256 x 64
-  if (m <= 128) return 1;  // 256 x 128
+int pick_tiled(int family, int64_t m, int64_t np) {
+  if (m <= 32) return 4;   // 256 x 32, register-staged
+  if (m <= 64) return 3;   // 256 x 64, register-staged
+  if (m <= 128) return 9;  // 256 x 128, four-stage LDS ring
   const int64_t tiles256 = ((np + 255) / 256) * ((m + 255) / 256);
-  if (tiles256 < 192) return 2;  // 128 x 128
-  return 0;                      // 256 x 256
+  if (tiles256 < 192) return 7;  // 128 x 128, direct-to-LDS
+  // 256 x 256: the gate/up product runs best on the four-stage ring, the deep-K down product on two stages
+  return family == 0 ? 8 : 5;
 }
 
 int resolve_variant(int family, int64_t m, int64_t np) {
   const int forced = g_forced_variant[family];
   if (forced >= 0 && !(forced == VARIANT_SKINNY && m > 64)) return forced;
   if (m <= 16) return VARIANT_SKINNY;  // decode: weight streaming, HBM bound
-  return pick_tiled(m, np);
+  return pick_tiled(family, m, np);
 }
 
 int finish(hipError_t e) {

@@ -24,7 +24,7 @@ struct TiledVariant {
   int bp, bq;        // workgroup tile: weight rows x activation rows
   int threads;
 };
-void set_raster_group(int g);  // activation-row tiles per raster band (tuning)
+void set_raster_group(int g);  // activation-row tiles per raster band; 0 restores the per-kernel default
 int tiled_variant_count();
 const TiledVariant& tiled_variant(int variant);
 hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, hipStream_t stream);

@@ -17,6 +17,8 @@
 // row r is stored at chunk position c ^ (r & 7). A wave's ds_read_b128 for an MFMA operand touches 32
 // consecutive rows at one logical chunk (x2 for the two K halves), so any 8 consecutive lanes cover all 32
 // banks exactly once; the global->LDS copy writes whole 128-byte rows per 8 lanes. Both are conflict-free.
+#include <type_traits>
+
 #include "fsw_internal.h"
 #include "fsw_device.h"
 
@@ -420,6 +422,214 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
   store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
 }
 
+// ---- four-stage direct-to-LDS variant ------------------------------------------------------------------------
+// K tiles of 32 elements in a ring of four LDS stages: the DMA of tile kt+3 is issued while tile kt is being
+// multiplied, so a copy has three iterations (~3000 MFMA cycles) to land instead of one. That covers L2 misses
+// (Infinity Cache / HBM latency), which the two-stage kernels above expose at every barrier.
+// LDS rows are 64 bytes (4 chunks of 16 B); chunk c of row r sits at position c ^ ((r >> 2) & 3): 16 consecutive
+// rows at one logical chunk then cover the 64 banks once. The barrier waits for this wave's copy of tile kt+1
+// only (vmcnt leaves the two younger tiles in flight), hence the hand-written s_waitcnt.
+template <class E, bool GATED, bool KTAIL, int WP, int WQ, int FP, int FQ>
+__global__ void __launch_bounds__(WP* WQ * 64)
+tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
+  constexpr int NT = WP * WQ * 64;
+  constexpr int BP = WP * FP * 32;
+  constexpr int BQ = WQ * FQ * 32;
+  constexpr int BK = 32;
+  constexpr int ROWB = BK * 2;      // 64
+  constexpr int RSTEP = NT / 4;     // rows covered by one round of DMA instructions (16 rows per wave)
+  constexpr int LP = BP / RSTEP;
+  constexpr int LQ = BQ / RSTEP;
+  constexpr int NL = LP + LQ;       // DMA instructions per wave per K tile
+  constexpr int STAGE = (BP + BQ) * ROWB;
+  static_assert(BP % RSTEP == 0 && BQ % RSTEP == 0 && RSTEP % 16 == 0, "copy mapping");
+  static_assert(!GATED || (FP % 2 == 0), "gated kernel pairs fragments");
+  static_assert(4 * STAGE <= 160 * 1024, "LDS budget of a gfx950 CU");
+  static_assert(2 * NL <= 63, "vmcnt is a 6-bit counter");
+
+  __shared__ __align__(1024) unsigned char ring0[STAGE];
+  __shared__ __align__(1024) unsigned char ring1[STAGE];
+  __shared__ __align__(1024) unsigned char ring2[STAGE];
+  __shared__ __align__(1024) unsigned char ring3[STAGE];
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wq = wave % WQ;
+  const int wp = wave / WQ;
+  const int l32 = lane & 31;
+  const int hi = lane >> 5;
+
+  int tp, tq;
+  tile_coords(blockIdx.x, tiles_p, tiles_q, group, tp, tq);
+  const int p0 = tp * BP;
+  const int q0 = tq * BQ;
+
+  const int pc = t & 3;
+  const int rb = t >> 2;
+  const int lc = pc ^ ((rb >> 2) & 3);
+  const unsigned char* pbase = (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
+  const unsigned char* qbase = (const unsigned char*)a.Q + (long long)q0 * a.ldq * 2;
+  const __amdgpu_buffer_rsrc_t prs = make_rsrc(pbase, ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
+  const __amdgpu_buffer_rsrc_t qrs = make_rsrc(qbase, ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2);
+  unsigned poff[LP], qoff[LQ];
+#pragma unroll
+  for (int i = 0; i < LP; ++i) {
+    const int r = rb + i * RSTEP;
+    const int grow = GATED ? (r < BP / 2 ? 2 * r : 2 * (r - BP / 2) + 1) : r;
+    poff[i] = (unsigned)grow * (unsigned)a.ldp * 2u + (unsigned)lc * 16u;
+  }
+#pragma unroll
+  for (int i = 0; i < LQ; ++i) {
+    const int r = rb + i * RSTEP;
+    qoff[i] = (unsigned)r * (unsigned)a.ldq * 2u + (unsigned)lc * 16u;
+  }
+
+  unsigned xo[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) xo[ks] = (unsigned)((((ks << 1) | hi) ^ ((l32 >> 2) & 3)) * 16);
+  const unsigned rd_p = (unsigned)((GATED ? wp * (FP / 2) * 32 : wp * FP * 32) + l32) * ROWB;
+  const unsigned rd_q = (unsigned)(BP + wq * FQ * 32 + l32) * ROWB;
+  auto p_frag_off = [](int f) -> unsigned {
+    if (GATED) return (unsigned)((f < FP / 2 ? f * 32 : BP / 2 + (f - FP / 2) * 32) * ROWB);
+    return (unsigned)(f * 32 * ROWB);
+  };
+
+  f32x16 acc[FP][FQ];
+#pragma unroll
+  for (int f = 0; f < FP; ++f)
+#pragma unroll
+    for (int g = 0; g < FQ; ++g)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[f][g][i] = 0.0f;
+
+  const int nkt = (a.k + BK - 1) / BK;
+
+  // DMA instructions lo..hi-1 (of NL per wave: weight rows first, then activation rows) of K tile `kt`.
+  auto dma = [&](unsigned char* stage, int kt, auto lo_c, auto hi_c) {
+    constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
+    const int ktc = kt < nkt ? kt : nkt - 1;  // past the end: re-read the last tile, never consumed
+    const int kb = ktc * (BK * 2);
+    const bool in = !KTAIL || (ktc * BK + lc * 8) < a.k;
+#pragma unroll
+    for (int i = LO; i < HI; ++i) {
+      if (i < LP) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(stage + i * RSTEP * ROWB + wave * 1024), 16,
+                                                 (int)(in ? poff[i] : OOB_OFFSET), kb, 0, 0);
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(stage + (BP + (i - LP) * RSTEP) * ROWB + wave * 1024),
+                                                 16, (int)(in ? qoff[i - LP] : OOB_OFFSET), kb, 0, 0);
+      }
+    }
+  };
+  auto dma_all = [&](unsigned char* stage, int kt) {
+    dma(stage, kt, std::integral_constant<int, 0>{}, std::integral_constant<int, NL>{});
+  };
+
+  u32x4 pf[2][FP], qf[2][FQ];
+  auto f_read = [&](int fb, const unsigned char* base, int ks) {
+    pf[fb][0] = *(const u32x4*)(base + rd_p + p_frag_off(0) + xo[ks]);
+#pragma unroll
+    for (int g = 0; g < FQ; ++g) qf[fb][g] = *(const u32x4*)(base + rd_q + g * 32 * ROWB + xo[ks]);
+#pragma unroll
+    for (int f = 1; f < FP; ++f) pf[fb][f] = *(const u32x4*)(base + rd_p + p_frag_off(f) + xo[ks]);
+  };
+  auto mma = [&](int fb, int f_lo, int f_hi) {
+#pragma unroll
+    for (int f = f_lo; f < f_hi; ++f)
+#pragma unroll
+      for (int g = 0; g < FQ; ++g) acc[f][g] = E::mfma32(pf[fb][f], qf[fb][g], acc[f][g]);
+  };
+
+  constexpr int NM = FP * FQ;
+  constexpr int NR = FP + FQ;
+  constexpr int HF = FP / 2 > 0 ? FP / 2 : 1;
+  constexpr int MPR = NM / NR > 0 ? NM / NR : 1;
+  // The NL copies of a K tile are issued in three parts spread over the iteration (a burst fills the texture
+  // addresser's queue and stalls the wave, and with it the MFMA stream): DA in step 0, DB in the first half of
+  // step 1, DC after the barrier.
+  constexpr int DA = NL / 2, DB = (NL - DA) / 2, DC = NL - DA - DB;
+  using C0 = std::integral_constant<int, 0>;
+  using CA = std::integral_constant<int, DA>;
+  using CB = std::integral_constant<int, DA + DB>;
+  using CN = std::integral_constant<int, NL>;
+  // s_waitcnt vmcnt(VM) lgkmcnt(0): this wave's copy of the next tile has landed (everything younger stays in
+  // flight: the tile after it and parts A and B of the one after that) and its own LDS reads are complete; then
+  // the workgroup barrier publishes every wave's part.
+  constexpr int VM = NL + DA + DB;
+  static_assert(VM <= 63, "vmcnt is a 6-bit counter");
+  constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
+  auto ring_barrier = [&]() {
+    asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(WAIT_IMM) : "memory");
+  };
+
+  // One K tile: `cur` holds tile kt with its step-0 fragments already in pf[0]/qf[0]; `nxt` holds (or is about
+  // to hold) tile kt+1; `fill` is the stage every wave finished reading before the previous barrier.
+  auto iteration = [&](unsigned char* cur, unsigned char* nxt, unsigned char* fill, int kt) {
+    dma(fill, kt + 3, C0{}, CA{});
+    f_read(1, cur, 1);
+    mma(0, 0, FP);
+    if constexpr (FP == 4 && FQ == 4 && DA == 4) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, (DA + NR - 1) / NR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    }
+    dma(fill, kt + 3, CA{}, CB{});
+    mma(1, 0, HF);
+#pragma unroll
+    for (int i = 0; i < DB; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, (HF * FQ) / (DB > 0 ? DB : 1), 0);
+      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+    }
+    ring_barrier();
+    f_read(0, nxt, 0);
+    dma(fill, kt + 3, CB{}, CN{});
+    mma(1, HF, FP);
+    constexpr int MC = (FP - HF) * FQ;  // MFMAs after the barrier
+#pragma unroll
+    for (int j = 0; j < (DC > 0 ? DC : 1); ++j) {
+#pragma unroll
+      for (int i = 0; i < MC / (DC > 0 ? DC : 1); ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, (NR + MC - 1) / MC, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x010, DC > 0 ? 1 : 0, 0);
+    }
+  };
+
+  if (nkt > 0) {
+    dma_all(ring0, 0);
+    dma_all(ring1, 1);
+    dma_all(ring2, 2);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NL) : "memory");  // tile 0 landed, tiles 1 and 2 pending
+    f_read(0, ring0, 0);
+  }
+  int kt = 0;
+  for (; kt + 3 < nkt; kt += 4) {
+    iteration(ring0, ring1, ring3, kt);
+    iteration(ring1, ring2, ring0, kt + 1);
+    iteration(ring2, ring3, ring1, kt + 2);
+    iteration(ring3, ring0, ring2, kt + 3);
+  }
+  if (kt < nkt) iteration(ring0, ring1, ring3, kt++);
+  if (kt < nkt) iteration(ring1, ring2, ring0, kt++);
+  if (kt < nkt) iteration(ring2, ring3, ring1, kt++);
+
+  store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
+}
+
 // ---- variant table ------------------------------------------------------------------------------------
 namespace {
 
@@ -432,9 +642,18 @@ const TiledVariant kVariants[] = {
     {"dma_256x256", 256, 256, 256},    // direct-to-LDS copies, conflict-free operand reads
     {"dma_256x128", 256, 128, 256},
     {"dma_128x128", 128, 128, 256},
+    {"ring_256x256", 256, 256, 256},   // four-stage LDS ring, K tiles of 32
+    {"ring_256x128", 256, 128, 256},
+    {"ring8w_256x256_a", 256, 256, 512},  // 8 waves (2 per SIMD), wave tile 128 x 64
+    {"ring8w_256x256_b", 256, 256, 512},  // 8 waves, wave tile 64 x 128
+    {"dma8w_256x256", 256, 256, 512},
 };
 
-int g_raster_group = 4;
+int g_raster_group = 0;  // 0 = per-launch default
+
+// Activation-row tiles per raster band. Measured on the headline shapes: the gate/up product (many weight
+// panels, 4096-deep K) prefers 4, the down product (few weight panels, 14336-deep K) prefers 2.
+int raster_group(bool gated) { return g_raster_group > 0 ? g_raster_group : (gated ? 4 : 2); }
 
 template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
 hipError_t launch_one(const GemmArgs& a, hipStream_t stream) {
@@ -443,7 +662,7 @@ hipError_t launch_one(const GemmArgs& a, hipStream_t stream) {
   const int tiles_q = (a.nq + BQ - 1) / BQ;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
   hipLaunchKernelGGL((tiled_kernel<E, GATED, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)), dim3(WP * WQ * 64), 0,
-                     stream, a, tiles_p, tiles_q, g_raster_group);
+                     stream, a, tiles_p, tiles_q, raster_group(GATED));
   return hipGetLastError();
 }
 
@@ -455,10 +674,26 @@ hipError_t launch_dma(const GemmArgs& a, hipStream_t stream) {
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
   if (a.k % 64 == 0) {
     hipLaunchKernelGGL((tiled_dma_kernel<E, GATED, false, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
-                       dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, g_raster_group);
+                       dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, raster_group(GATED));
   } else {
     hipLaunchKernelGGL((tiled_dma_kernel<E, GATED, true, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
-                       dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, g_raster_group);
+                       dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, raster_group(GATED));
+  }
+  return hipGetLastError();
+}
+
+template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
+hipError_t launch_ring(const GemmArgs& a, hipStream_t stream) {
+  constexpr int BP = WP * FP * 32, BQ = WQ * FQ * 32;
+  const int tiles_p = (a.np + BP - 1) / BP;
+  const int tiles_q = (a.nq + BQ - 1) / BQ;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  if (a.k % 32 == 0) {
+    hipLaunchKernelGGL((tiled_ring_kernel<E, GATED, false, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
+                       dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, raster_group(GATED));
+  } else {
+    hipLaunchKernelGGL((tiled_ring_kernel<E, GATED, true, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
+                       dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, raster_group(GATED));
   }
   return hipGetLastError();
 }
@@ -474,13 +709,18 @@ hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
     case 5: return launch_dma<E, GATED, 2, 2, 4, 4>(a, stream);
     case 6: return launch_dma<E, GATED, 2, 2, 4, 2>(a, stream);
     case 7: return launch_dma<E, GATED, 2, 2, 2, 2>(a, stream);
+    case 8: return launch_ring<E, GATED, 2, 2, 4, 4>(a, stream);
+    case 9: return launch_ring<E, GATED, 2, 2, 4, 2>(a, stream);
+    case 10: return launch_ring<E, GATED, 2, 4, 4, 2>(a, stream);
+    case 11: return launch_ring<E, GATED, 4, 2, 2, 4>(a, stream);
+    case 12: return launch_dma<E, GATED, 2, 4, 4, 2>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
 }  // namespace
 
-void set_raster_group(int g) { g_raster_group = g > 0 ? g : 4; }
+void set_raster_group(int g) { g_raster_group = g > 0 ? g : 0; }
 int tiled_variant_count() { return (int)(sizeof(kVariants) / sizeof(kVariants[0])); }
 const TiledVariant& tiled_variant(int variant) { return kVariants[variant]; }
 

@@ -113,9 +113,10 @@ FSW_API int fsw_last_hip_error(void);
 FSW_API int fsw_version(void);
 
 /*
- * Kernel-selection override for tuning and tests. family: 0 = gate/up, 1 = down.
- * variant < 0 restores the automatic choice by shape. Returns FSW_E_VARIANT for unknown ids.
- * Process-wide and not thread-safe against concurrent launches.
+ * Kernel-selection override for tuning and tests. family: 0 = gate/up, 1 = down; variant < 0 restores the
+ * automatic choice by shape; variant 100 is the weight-streaming kernel (honoured for M <= 64).
+ * family 2 sets the raster band height of the tiled kernels instead (0 = per-kernel default).
+ * Returns FSW_E_VARIANT for unknown ids. Process-wide and not thread-safe against concurrent launches.
  */
 FSW_API int fsw_set_variant(int family, int variant);
 
