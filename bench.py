@@ -28,6 +28,9 @@ sys.path.insert(0, os.path.join(ROOT, "fused-swiglu_amd"))
 
 MFMA_PEAK_TFLOPS = 2516.6  # MI355X dense bf16/fp16: 256 CU x 2.4 GHz x 4096 flop/clk/CU
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+# L2<->fabric bytes per launch of the dominant kernel, from separate `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
+# runs scaled by a 1 GiB copy kernel (profiles/tiled_prefill_C3_hbm_traffic_pmc.md); not measurable in-process.
+MEASURED_TRAFFIC_BYTES = {"C3": 2753080 * 1024 + 229388 * 1024}
 
 
 def parse():
@@ -39,6 +42,10 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the cpu_baseline sample")
     ap.add_argument("--detail", action="store_true", help="also time every configuration (stderr table)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one elementwise copy of 1 GiB (reads 1 GiB, writes 1 GiB): the known-size kernel "
+                         "that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
+    ap.add_argument("--no-decode", action="store_true", help="skip the M=16 decode leg")
     return ap.parse_args()
 
 
@@ -154,8 +161,9 @@ def main():
     else:
         roofline = {"bound": "mfma", "kernel": capi.variant_name(0, 0, M, 2 * ff, d) + " (gate/up)",
                     "achieved": round(gu_tflops, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(gu_tflops / MFMA_PEAK_TFLOPS, 4), "traffic": None,
-                    "avg_kernel_ms": round(gu_ms, 5)}
+                    "frac": round(gu_tflops / MFMA_PEAK_TFLOPS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    "algorithmic_bytes": (2 * ff * d + M * d + M * ff) * 2, "avg_kernel_ms": round(gu_ms, 5)}
     out = {
         "metric": "fused SwiGLU fwd TFLOP/s + % bf16 MFMA peak (M=8192,d=4096,ff=14336)",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -172,10 +180,18 @@ def main():
     }
 
     # decode leg: M = 16, weight streaming, judged in GB/s
-    if args.workload != "C4":
+    if args.copy_probe:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+
+    if args.workload != "C4" and not args.no_decode:
         inp4, g4 = load("C4")
         c4 = {k: inp4[k] for k in ("name", "M", "d", "ff", "seed")}
-        wall4, gu4, dn4, _ = run_steps(capi, torch, g4, c4, 200, 20)
+        wall4, _, _, _ = run_steps(capi, torch, g4, c4, 200, 20, with_events=False)  # step time: no events between launches
+        _, gu4, dn4, _ = run_steps(capi, torch, g4, c4, 100, 5)                       # per-kernel durations
         ms4 = wall4 / 200 * 1e3
         by4 = fsw_weights.hbm_bytes(c4["M"], c4["d"], c4["ff"])
         out["decode"] = {"workload": "C4: M=16 d=4096 ff=14336 bf16 seed 3", "ms_per_step": round(ms4, 5),
