@@ -13,6 +13,7 @@ thread_local int g_last_hip_error = 0;
 int g_forced_variant[2] = {-1, -1};  // family 0 = gate/up, 1 = down
 
 constexpr int VARIANT_SKINNY = 100;          // id of the weight-streaming kernel in fsw_set_variant
+constexpr int VARIANT_DECODE_FUSED = 101;    // fsw_mlp only: single-launch decode forward (family 0)
 constexpr int64_t MAX_DIM = 1LL << 30;       // every size is cast to int inside the kernels
 constexpr int64_t MAX_LD = 1LL << 21;        // keeps tile-relative byte offsets below 2^31
 
@@ -54,6 +55,7 @@ int pick_tiled(int family, int64_t m, int64_t np) {
 
 int resolve_variant(int family, int64_t m, int64_t np) {
   const int forced = g_forced_variant[family];
+  if (forced == VARIANT_DECODE_FUSED) return m <= 16 ? VARIANT_SKINNY : pick_tiled(family, m, np);
   if (forced >= 0 && !(forced == VARIANT_SKINNY && m > 64)) return forced;
   if (m <= 16) return VARIANT_SKINNY;  // decode: weight streaming, HBM bound
   return pick_tiled(family, m, np);
@@ -97,7 +99,9 @@ int fsw_set_variant(int family, int variant) {
     return FSW_OK;
   }
   if (family < 0 || family > 1) return FSW_E_VARIANT;
-  if (variant >= 0 && variant != VARIANT_SKINNY && variant >= fsw::tiled_variant_count()) return FSW_E_VARIANT;
+  if (variant >= 0 && variant != VARIANT_SKINNY && !(family == 0 && variant == VARIANT_DECODE_FUSED) &&
+      variant >= fsw::tiled_variant_count())
+    return FSW_E_VARIANT;
   g_forced_variant[family] = variant < 0 ? -1 : variant;
   return FSW_OK;
 }
@@ -222,6 +226,28 @@ int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t 
   rc = fsw_validate_down(dtype, M, D, FF, Hbuf, FF, W2, ldw2, Y, ldy);
   if (rc != FSW_OK) return rc;
   if (M == 0 || D == 0) return FSW_OK;
+  if (M <= 16 && FF > 0 && g_forced_variant[0] == VARIANT_DECODE_FUSED) {
+    // opt-in: one persistent launch does both projections with a device-wide barrier in between. Measured
+    // slower than the two weight-streaming launches so far (stragglers before the barrier), so not the default.
+    fsw::DecodeArgs da;
+    da.X = X;
+    da.W13 = W13;
+    da.W2 = W2;
+    da.H = Hbuf;
+    da.Y = Y;
+    da.ldx = ldx;
+    da.ldw13 = ldw13;
+    da.ldw2 = ldw2;
+    da.ldy = ldy;
+    da.nq = (int)M;
+    da.d = (int)D;
+    da.ff = (int)FF;
+    if (fsw::decode_mlp_supported(da)) {
+      const int drc = check_device();
+      if (drc != FSW_OK) return drc;
+      return finish(fsw::launch_decode_mlp(dtype, da, (hipStream_t)stream));
+    }
+  }
   rc = fsw_gateup(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF, stream);
   if (rc != FSW_OK) return rc;
   unsigned char* ws2 = (unsigned char*)workspace + h_bytes(M, FF);

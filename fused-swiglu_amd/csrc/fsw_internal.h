@@ -38,3 +38,21 @@ SkinnyPlan skinny_plan(bool gated, int np, int nq, int k);
 hipError_t launch_skinny(int dtype, bool gated, const GemmArgs& a, void* workspace, hipStream_t stream);
 
 }  // namespace fsw
+
+namespace fsw {
+
+// Single-launch decode forward (kernels_decode.hip): gate/up, device-wide barrier, down projection, for at most
+// 16 activation rows. H is a caller-provided [nq, ff] scratch matrix (row stride ff).
+struct DecodeArgs {
+  const void* X;
+  const void* W13;
+  const void* W2;
+  void* H;
+  void* Y;
+  long long ldx, ldw13, ldw2, ldy;  // elements
+  int nq, d, ff;
+};
+bool decode_mlp_supported(const DecodeArgs& a);
+hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream);
+
+}  // namespace fsw

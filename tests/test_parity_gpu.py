@@ -139,6 +139,35 @@ def test_skinny_weight_streaming_variant(capi, M, dtype):
         capi.set_variant(1, -1)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [1, 5, 16])
+def test_single_launch_decode_forward(capi, M, dtype):
+    """With variant 101 fsw_mlp runs M <= 16 as one launch (gate/up, device-wide barrier, down projection); it
+    must agree with the two-launch path and with the oracle, call after call (the barrier slots restore
+    themselves) and for ragged d / ff."""
+    for (d, ff) in [(8, 8), (136, 40), (1000, 264), (4096, 1032), (512, 14336), (4096, 14336)]:
+        inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=77 * M + d, x_scale=0.5)
+        g = to_dev(inp)
+        ws = capi.mlp_workspace(g["X"], ff)
+        try:
+            capi.set_variant(0, 101)
+            Y1 = capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws)
+            H1 = ws[: M * ff * 2].view(dtype).view(M, ff).clone()
+            reps = [capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws) for _ in range(3)]  # barrier slots are reused
+        finally:
+            capi.set_variant(0, -1)
+        Y2 = capi.mlp(g["X"], g["W13"], g["W2"])
+        H2 = capi.gateup(g["X"], g["W13"])
+        assert_one_rounding(H1, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "fused H %s" % ((M, d, ff),))
+        assert_one_rounding(Y1, oracle.ref_down(H1.cpu(), inp["W2"], torch.float64), dtype, "fused Y|H %s" % ((M, d, ff),))
+        oracle.assert_parity(Y1, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64), "fused mlp %s" % ((M, d, ff),))
+        # the two paths differ only in fp32 summation order
+        assert (H1.float() - H2.float()).abs().max().item() <= 2 * ulp_rel(dtype) * 2 * H2.float().abs().max().item() + 1e-3
+        assert (Y1.float() - Y2.float()).abs().max().item() <= 2e-2
+        for r in reps:
+            assert torch.equal(r, Y1)
+
+
 def test_empty_and_degenerate_problems(capi):
     bf = torch.bfloat16
     X = torch.randn(0, 64, device=DEV).to(bf)
