@@ -44,20 +44,17 @@ int check_device() {
 // Variant choice for the tiled kernels: the widest tile whose activation-row extent is not mostly padding,
 // stepping down to 128x128 when a 256-wide grid would leave most of the 256 CUs idle.
 int pick_tiled(int family, int64_t m, int64_t np) {
-  if (m <= 32) return 4;   // 256 x 32, register-staged
-  if (m <= 64) return 3;   // 256 x 64, register-staged
-  if (m <= 128) return 9;  // 256 x 128, four-stage LDS ring
   const int64_t tiles256 = ((np + 255) / 256) * ((m + 255) / 256);
-  if (tiles256 < 192) return 7;  // 128 x 128, direct-to-LDS
+  if (tiles256 < 192) return 7;  // 128 x 128, direct-to-LDS (with split-K for the down product, see fsw_down)
   // 256 x 256: the gate/up product runs best on the four-stage ring, the deep-K down product on two stages
   return family == 0 ? 8 : 5;
 }
 
 int resolve_variant(int family, int64_t m, int64_t np) {
   const int forced = g_forced_variant[family];
-  if (forced == VARIANT_DECODE_FUSED) return m <= 16 ? VARIANT_SKINNY : pick_tiled(family, m, np);
+  if (forced == VARIANT_DECODE_FUSED) return m <= 64 ? VARIANT_SKINNY : pick_tiled(family, m, np);
   if (forced >= 0 && !(forced == VARIANT_SKINNY && m > 64)) return forced;
-  if (m <= 16) return VARIANT_SKINNY;  // decode: weight streaming, HBM bound
+  if (m <= 64) return VARIANT_SKINNY;  // decode and small batches: weight streaming, HBM bound
   return pick_tiled(family, m, np);
 }
 
@@ -171,10 +168,9 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
 
 size_t fsw_down_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
   (void)dtype;
-  (void)M;
-  (void)D;
-  (void)FF;
-  return 0;
+  if (M <= 64 || M > MAX_DIM || D <= 0 || D > MAX_DIM || FF <= 0 || FF > MAX_DIM) return 0;
+  const fsw::SplitPlan plan = fsw::tiled_split_plan((int)D, (int)M, (int)FF);
+  return plan.splits > 1 ? (size_t)plan.splits * (size_t)M * (size_t)D * sizeof(float) : 0;
 }
 
 int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t ldh, const void* W2, int64_t ldw2,
@@ -198,6 +194,13 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
   a.k = (int)FF;
   const int v = resolve_variant(1, M, D);
   if (v == VARIANT_SKINNY) return finish(fsw::launch_skinny(dtype, false, a, workspace, (hipStream_t)stream));
+  if (need > 0 && g_forced_variant[1] < 0) {  // few output tiles, deep K: split K across workgroups
+    if (!aligned16(workspace)) return FSW_E_ALIGN;
+    const fsw::SplitPlan plan = fsw::tiled_split_plan((int)D, (int)M, (int)FF);
+    a.splits = plan.splits;
+    a.partial = (float*)workspace;
+    return finish(fsw::launch_tiled_splitk(dtype, plan.tile, a, (hipStream_t)stream));
+  }
   return finish(fsw::launch_tiled(v, dtype, false, a, (hipStream_t)stream));
 }
 

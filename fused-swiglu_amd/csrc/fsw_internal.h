@@ -16,6 +16,10 @@ struct GemmArgs {
   void* O;
   long long ldp, ldq, ldo;  // elements
   int np, nq, k;
+  // split-K (plain kernel only): `splits` workgroups share one output tile, each over a contiguous K range, and
+  // store fp32 partial sums to partial[split][nq][np]; splitk_reduce() sums them and rounds once.
+  int splits = 1;
+  float* partial = nullptr;
 };
 
 // Tiled LDS/MFMA kernels (kernels_tiled.hip). `variant` indexes tiled_variant_table().
@@ -28,6 +32,15 @@ void set_raster_group(int g);  // activation-row tiles per raster band; 0 restor
 int tiled_variant_count();
 const TiledVariant& tiled_variant(int variant);
 hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
+// Plan for the plain (down-projection) product when the output has few tiles and K is deep: which direct-to-LDS
+// tile (128 or 256 square) and how many K partitions, so that about two workgroups per CU are in flight.
+// splits == 1 means the ordinary launch path.
+struct SplitPlan {
+  int tile;    // 128 or 256
+  int splits;  // K partitions
+};
+SplitPlan tiled_split_plan(int np, int nq, int k);
+hipError_t launch_tiled_splitk(int dtype, int tile, const GemmArgs& a, hipStream_t stream);  // a.splits, a.partial set
 
 // Weight-streaming kernels for M <= 16 activation rows (kernels_skinny.hip).
 struct SkinnyPlan {

@@ -68,6 +68,71 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[FP][FQ], const GemmArgs
   }
 }
 
+// Split-K epilogue of the plain kernel: fp32 partial sums to partial[split][m][n], 16 bytes per lane.
+template <int WP, int WQ, int FP, int FQ>
+__device__ __forceinline__ void store_partial(f32x16 (&acc)[FP][FQ], const GemmArgs& a, int split, int p0, int q0,
+                                              int wp, int wq, int l32, int hi) {
+  float* base = a.partial + (long long)split * a.nq * a.np;
+#pragma unroll
+  for (int g = 0; g < FQ; ++g) {
+    const int m = q0 + (wq * FQ + g) * 32 + l32;
+    if (m >= a.nq) continue;
+    float* row = base + (long long)m * a.np;
+#pragma unroll
+    for (int f = 0; f < FP; ++f) {
+      const int nb = p0 + (wp * FP + f) * 32 + hi * 4;
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int n = nb + i4 * 8;
+        if (((a.np & 3) == 0) && n + 3 < a.np) {
+          f32x4 v = {acc[f][g][i4 * 4], acc[f][g][i4 * 4 + 1], acc[f][g][i4 * 4 + 2], acc[f][g][i4 * 4 + 3]};
+          *(f32x4*)(row + n) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < a.np) row[n + e] = acc[f][g][i4 * 4 + e];
+        }
+      }
+    }
+  }
+}
+
+// O[m, n] = round(sum over splits of partial[s][m][n]); one thread per 4 consecutive n.
+template <class E>
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(const float* __restrict__ partial, int splits, int nq, int np, unsigned short* __restrict__ O,
+                     long long ldo) {
+  const int groups = (np + 3) >> 2;
+  const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (long long)nq * groups) return;
+  const int m = (int)(id / groups);
+  const int n = (int)(id - (long long)m * groups) * 4;
+  const long long plane = (long long)nq * np;
+  const float* src = partial + (long long)m * np + n;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool full = ((np & 3) == 0) && n + 3 < np;
+  for (int s = 0; s < splits; ++s) {
+    if (full) {
+      const f32x4 t = *(const f32x4*)(src + s * plane);
+      v[0] += t[0];
+      v[1] += t[1];
+      v[2] += t[2];
+      v[3] += t[3];
+    } else {
+      for (int e = 0; e < 4; ++e)
+        if (n + e < np) v[e] += src[s * plane + e];
+    }
+  }
+  unsigned short* orow = O + (long long)m * ldo;
+  if (full && ((ldo & 3) == 0) && ((((uintptr_t)O) & 7) == 0)) {
+    u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
+    *(u32x2*)(orow + n) = pk;
+  } else {
+    for (int e = 0; e < 4; ++e)
+      if (n + e < np) orow[n + e] = E::cvt1(v[e]);
+  }
+}
+
 template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
 __global__ void __launch_bounds__(WP* WQ * 64)
 tiled_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
@@ -330,14 +395,18 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[f][g][i] = 0.0f;
 
-  const int nkt = (a.k + BK - 1) / BK;
+  // K range of this workgroup: everything, or one of a.splits contiguous runs of K tiles (blockIdx.y)
+  const int nkt_all = (a.k + BK - 1) / BK;
+  const int kt_per = (nkt_all + a.splits - 1) / a.splits;
+  const int kt0 = (int)blockIdx.y * kt_per;
+  const int nkt = nkt_all - kt0 < kt_per ? (nkt_all - kt0 > 0 ? nkt_all - kt0 : 0) : kt_per;
 
   // DMA of K tile `kt` into `stage`: wave-uniform LDS base per instruction, loop-invariant per-lane offset in a
   // VGPR, the K offset in an SGPR. Rows beyond the matrix are out of range for the buffer descriptor and arrive
   // as zeros. A prefetch past the last tile re-reads the last tile (never consumed). Only when K is not a
   // multiple of 64 (KTAIL) do lanes whose chunk lies at or beyond K redirect their offset out of range.
   auto dma = [&](unsigned char* stage, int kt) {
-    const int ktc = kt < nkt ? kt : nkt - 1;
+    const int ktc = kt0 + (kt < nkt ? kt : nkt - 1);
     const int kb = ktc * (BK * 2);
     const bool in = !KTAIL || (ktc * BK + lc * 8) < a.k;
 #pragma unroll
@@ -419,6 +488,12 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
   }
   if (kt < nkt) iteration(lds0, lds1, kt);
 
+  if constexpr (!GATED) {
+    if (a.splits > 1) {
+      store_partial<WP, WQ, FP, FQ>(acc, a, (int)blockIdx.y, p0, q0, wp, wq, l32, hi);
+      return;
+    }
+  }
   store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
 }
 
@@ -719,6 +794,61 @@ hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
 }
 
 }  // namespace
+
+SplitPlan tiled_split_plan(int np, int nq, int k) {
+  const long long t128 = (long long)((np + 127) / 128) * ((nq + 127) / 128);
+  const long long t256 = (long long)((np + 255) / 256) * ((nq + 255) / 256);
+  SplitPlan p = {256, 1};
+  if (t128 <= 0 || t256 >= 192) return p;
+  int by_k;
+  long long tiles;
+  if (t128 < 256) {
+    p.tile = 128;
+    tiles = t128;
+    by_k = k / 512;  // at least 8 K tiles of 64 per partition
+  } else {
+    tiles = t256;
+    by_k = k / 1024;
+  }
+  int splits = (int)((512 + tiles - 1) / tiles);
+  if (splits > by_k) splits = by_k;
+  if (splits > 16) splits = 16;
+  p.splits = splits < 1 ? 1 : splits;
+  if (p.splits == 1 && p.tile == 256) p.tile = 128;  // unsplit mid-size problems keep the smaller tile
+  return p;
+}
+
+namespace {
+template <class E, int WP, int WQ, int FP, int FQ>
+hipError_t launch_splitk_one(const GemmArgs& a, hipStream_t stream) {
+  constexpr int BP = WP * FP * 32, BQ = WQ * FQ * 32;
+  const int tiles_p = (a.np + BP - 1) / BP;
+  const int tiles_q = (a.nq + BQ - 1) / BQ;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  const dim3 grid((unsigned)(tiles_p * tiles_q), (unsigned)a.splits);
+  const int group = raster_group(false);
+  if (a.k % 64 == 0) {
+    hipLaunchKernelGGL((tiled_dma_kernel<E, false, false, WP, WQ, FP, FQ>), grid, dim3(WP * WQ * 64), 0, stream, a,
+                       tiles_p, tiles_q, group);
+  } else {
+    hipLaunchKernelGGL((tiled_dma_kernel<E, false, true, WP, WQ, FP, FQ>), grid, dim3(WP * WQ * 64), 0, stream, a,
+                       tiles_p, tiles_q, group);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || a.splits <= 1) return e;
+  const long long work = (long long)a.nq * ((a.np + 3) / 4);
+  hipLaunchKernelGGL((splitk_reduce_kernel<E>), dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, a.partial,
+                     a.splits, a.nq, a.np, (unsigned short*)a.O, a.ldo);
+  return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_tiled_splitk(int dtype, int tile, const GemmArgs& a, hipStream_t stream) {
+  if (tile == 128) {
+    return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 2>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 2>(a, stream);
+  }
+  return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 4, 4>(a, stream) : launch_splitk_one<Fp16, 2, 2, 4, 4>(a, stream);
+}
 
 void set_raster_group(int g) { g_raster_group = g > 0 ? g : 0; }
 int tiled_variant_count() { return (int)(sizeof(kVariants) / sizeof(kVariants[0])); }

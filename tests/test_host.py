@@ -106,7 +106,13 @@ def test_variant_choice_by_regime(capi):
     assert "256x256" in name(0, 4096, 22016, 4096)
     assert name(0, 512, 5632, 1024) == "dma_128x128"     # small problem: more, smaller tiles
     assert name(0, 16, 28672, 4096) == "skinny" and name(1, 1, 4096, 14336) == "skinny"
-    assert name(0, 100, 28672, 4096) == "ring_256x128"
+    assert name(0, 64, 28672, 4096) == "skinny" and name(1, 33, 4096, 14336) == "skinny"
+    assert name(0, 100, 28672, 4096) == "dma_128x128"
+    # the down product with few output tiles and a deep K asks for split-K scratch; large or tiny M does not
+    ws = capi.lib().fsw_down_workspace_bytes
+    assert ws(0, 256, 4096, 14336) == 8 * 256 * 4096 * 4
+    assert ws(0, 8192, 4096, 14336) == 0 and ws(0, 16, 4096, 14336) == 0
+    assert capi.lib().fsw_mlp_workspace_bytes(0, 256, 4096, 14336) == 256 * 14336 * 2 + ws(0, 256, 4096, 14336)
 
 
 def test_packers_follow_the_reference_interleave():

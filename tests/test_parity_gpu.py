@@ -168,6 +168,37 @@ def test_single_launch_decode_forward(capi, M, dtype):
             assert torch.equal(r, Y1)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_split_k_down_projection(capi, dtype):
+    """65 <= M with few output tiles and a deep ff: fsw_down splits K across workgroups (fp32 partials in the
+    workspace, then one rounding). Checked against the oracle and, bit for bit up to summation order, against the
+    unsplit kernel."""
+    L = capi.lib()
+    for (M, d, ff) in [(200, 512, 4096), (130, 520, 2120), (65, 136, 8192), (256, 1024, 14336), (300, 264, 1032), (1024, 1024, 4096), (700, 2048, 2056)]:
+        inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=900 + M, x_scale=0.5)
+        g = to_dev(inp)
+        H = capi.gateup(g["X"], g["W13"])
+        nbytes = L.fsw_down_workspace_bytes(capi.dtype_code(H), M, d, ff)
+        Y = capi.down(H, g["W2"])
+        ref = oracle.ref_down(H.cpu(), inp["W2"], torch.float64)
+        assert_one_rounding(Y, ref, dtype, "split-K Y %s (scratch %d B)" % ((M, d, ff), nbytes))
+        try:
+            capi.set_variant(1, 7)  # same tile shape, no split
+            Y1 = capi.down(H, g["W2"])
+        finally:
+            capi.set_variant(1, -1)
+        assert (Y.float() - Y1.float()).abs().max().item() <= 4 * ulp_rel(dtype) * ref.abs().max().item() + 1e-3
+        assert torch.equal(capi.mlp(g["X"], g["W13"], g["W2"]), Y)
+    assert L.fsw_down_workspace_bytes(0, 200, 512, 4096) > 0 and L.fsw_down_workspace_bytes(0, 300, 264, 1032) > 0
+    # a missing or short workspace is refused, not ignored
+    inp = fsw_weights.make_inputs(200, 512, 4096, torch.bfloat16, seed=1)
+    g = to_dev(inp)
+    H = capi.gateup(g["X"], g["W13"])
+    Y = torch.empty(200, 512, dtype=torch.bfloat16, device=DEV)
+    rc = L.fsw_down(0, 200, 512, 4096, H.data_ptr(), 4096, g["W2"].data_ptr(), 4096, Y.data_ptr(), 512, None, 0, None)
+    assert rc == capi.E_WORKSPACE
+
+
 def test_empty_and_degenerate_problems(capi):
     bf = torch.bfloat16
     X = torch.randn(0, 64, device=DEV).to(bf)
