@@ -122,6 +122,33 @@ Tensor fused_swiglu_mlp_fp16(Tensor const& X, Tensor const& W1W3, Tensor const& 
   return fused_swiglu_mlp_typed(at::kHalf, X, W1W3, W2);
 }
 
+// ---- shape-only ("meta") implementations: let the ops trace under torch.compile / FakeTensor without a GPU.
+// The reference registers no such kernels and its swiglu_fwd_bf16 schema hides that C is written
+// (torch_bindings.cpp:42); `swiglu_fwd_bf16_out` below is the same call with the mutation declared.
+Tensor meta_gateup(at::ScalarType want, Tensor const& X, Tensor const& W1W3) {
+  TORCH_CHECK(X.scalar_type() == want, "Expected tensor A to be of type ", want, ", but got: ", X.scalar_type());
+  TORCH_CHECK(W1W3.scalar_type() == want, "Expected tensor B to be of type ", want, ", but got: ", W1W3.scalar_type());
+  TORCH_CHECK(X.dim() == 2 && W1W3.dim() == 2 && X.size(1) == W1W3.size(1) && W1W3.size(0) % 2 == 0,
+              "X is [M, K] and W1W3 is [2*ff, K]");
+  return at::empty({X.size(0), W1W3.size(0) / 2}, X.options());
+}
+Tensor meta_down(at::ScalarType want, Tensor const& H, Tensor const& W2) {
+  TORCH_CHECK(H.scalar_type() == want && W2.scalar_type() == want, "Expected tensors of type ", want);
+  TORCH_CHECK(H.dim() == 2 && W2.dim() == 2 && H.size(1) == W2.size(1), "H is [M, FF] and W2 is [D, FF]");
+  return at::empty({H.size(0), W2.size(0)}, H.options());
+}
+Tensor meta_fused_swiglu_bf16(Tensor const& X, Tensor const& W) { return meta_gateup(at::kBFloat16, X, W); }
+Tensor meta_fused_swiglu_fp16(Tensor const& X, Tensor const& W) { return meta_gateup(at::kHalf, X, W); }
+Tensor meta_down_bf16(Tensor const& H, Tensor const& W2) { return meta_down(at::kBFloat16, H, W2); }
+Tensor meta_down_fp16(Tensor const& H, Tensor const& W2) { return meta_down(at::kHalf, H, W2); }
+Tensor meta_mlp_bf16(Tensor const& X, Tensor const& W, Tensor const& W2) {
+  return meta_down(at::kBFloat16, meta_gateup(at::kBFloat16, X, W), W2);
+}
+Tensor meta_mlp_fp16(Tensor const& X, Tensor const& W, Tensor const& W2) {
+  return meta_down(at::kHalf, meta_gateup(at::kHalf, X, W), W2);
+}
+void meta_swiglu_fwd_bf16(int64_t, int64_t, int64_t, Tensor const&, int64_t, Tensor const&, int64_t, Tensor&, int64_t) {}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -147,6 +174,8 @@ TORCH_LIBRARY(ASMLLM, m) {
   m.def("swiglu_down_fp16(Tensor H, Tensor W2) -> Tensor");
   m.def("fused_swiglu_mlp_bf16(Tensor X, Tensor W1W3, Tensor W2) -> Tensor");
   m.def("fused_swiglu_mlp_fp16(Tensor X, Tensor W1W3, Tensor W2) -> Tensor");
+  // swiglu_fwd_bf16 with the write to C declared, for tracing compilers
+  m.def("swiglu_fwd_bf16_out(int m, int n, int k, Tensor A, int ldA, Tensor B, int ldB, Tensor(a!) C, int ldC) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(ASMLLM, CUDA, m) {
@@ -157,4 +186,16 @@ TORCH_LIBRARY_IMPL(ASMLLM, CUDA, m) {
   m.impl("swiglu_down_fp16", &swiglu_down_fp16);
   m.impl("fused_swiglu_mlp_bf16", &fused_swiglu_mlp_bf16);
   m.impl("fused_swiglu_mlp_fp16", &fused_swiglu_mlp_fp16);
+  m.impl("swiglu_fwd_bf16_out", &swiglu_fwd_bf16);
+}
+
+TORCH_LIBRARY_IMPL(ASMLLM, Meta, m) {
+  m.impl("fused_swiglu_bf16", &meta_fused_swiglu_bf16);
+  m.impl("fused_swiglu_fp16", &meta_fused_swiglu_fp16);
+  m.impl("swiglu_down_bf16", &meta_down_bf16);
+  m.impl("swiglu_down_fp16", &meta_down_fp16);
+  m.impl("fused_swiglu_mlp_bf16", &meta_mlp_bf16);
+  m.impl("fused_swiglu_mlp_fp16", &meta_mlp_fp16);
+  m.impl("swiglu_fwd_bf16", &meta_swiglu_fwd_bf16);
+  m.impl("swiglu_fwd_bf16_out", &meta_swiglu_fwd_bf16);
 }

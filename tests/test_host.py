@@ -185,3 +185,28 @@ def test_wrong_dtype_raises_runtime_error_like_the_reference(ext):
         ext.fused_swiglu_bf16(X32.bfloat16(), W32.bfloat16())
     with pytest.raises(RuntimeError):
         ext.fused_swiglu_bf16(torch.zeros(4, 8, dtype=torch.bfloat16), torch.zeros(6, 16, dtype=torch.bfloat16))
+
+
+def test_meta_kernels_trace_shapes_without_a_gpu(ext):
+    """Shape-only kernels registered under the Meta key: the ops can be traced by FakeTensor / torch.compile
+    front ends on a machine with no GPU. The mutation-annotated variant of swiglu_fwd_bf16 declares its write."""
+    X = torch.empty(33, 64, dtype=torch.bfloat16, device="meta")
+    W = torch.empty(80, 64, dtype=torch.bfloat16, device="meta")
+    W2 = torch.empty(64, 40, dtype=torch.bfloat16, device="meta")
+    H = torch.ops.ASMLLM.fused_swiglu_bf16(X, W)
+    assert H.shape == (33, 40) and H.dtype == torch.bfloat16 and H.device.type == "meta"
+    assert torch.ops.ASMLLM.swiglu_down_bf16(H, W2).shape == (33, 64)
+    assert torch.ops.ASMLLM.fused_swiglu_mlp_bf16(X, W, W2).shape == (33, 64)
+    assert torch.ops.ASMLLM.fused_swiglu_mlp_fp16(X.half(), W.half(), W2.half()).dtype == torch.float16
+    with pytest.raises(RuntimeError):
+        torch.ops.ASMLLM.fused_swiglu_bf16(X.half(), W.half())
+    with pytest.raises(RuntimeError):
+        torch.ops.ASMLLM.fused_swiglu_bf16(X, torch.empty(80, 32, dtype=torch.bfloat16, device="meta"))
+    schema = torch.ops.ASMLLM.swiglu_fwd_bf16_out.default._schema
+    assert schema.arguments[7].name == "C" and schema.arguments[7].alias_info is not None and schema.arguments[7].alias_info.is_write
+    assert not torch.ops.ASMLLM.swiglu_fwd_bf16.default._schema.arguments[7].alias_info  # the reference's schema, kept as is
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode():
+        a = torch.empty(5, 16, dtype=torch.bfloat16, device="cuda")
+        b = torch.empty(12, 16, dtype=torch.bfloat16, device="cuda")
+        assert torch.ops.ASMLLM.fused_swiglu_bf16(a, b).shape == (5, 6)
