@@ -69,6 +69,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, lo
 __device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
   return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
 }
+// Same load with the non-temporal cache policy: for weights that are read exactly once (decode). Measured on
+// the M=16 forward: 7 % faster than the default policy, which lets 353 MB of single-use lines churn through
+// the L2s and the 256 MB Infinity Cache and evict the activations that are reused.
+__device__ __forceinline__ u32x4 buf_load16_stream(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 2);
+}
 constexpr unsigned OOB_OFFSET = 0x80000000u;  // >= any num_records produced by make_rsrc
 
 // Workgroup id -> tile coordinates. Hardware deals consecutive workgroup ids round-robin over the 8 XCDs

@@ -78,7 +78,7 @@ __device__ __forceinline__ void decode_phase(const void* __restrict__ P, long lo
       const int lc = pc ^ row;  // slab chunk position pc of row `row` holds logical chunk pc ^ row (16 rows x 16 chunks)
       const bool in = live && (k0 + lc * 8) < k;
       const unsigned off = (unsigned)(p0 + row) * row_bytes + (unsigned)(k0 + lc * 8) * 2u;
-      w[i] = buf_load16(prs, in ? off : OOB_OFFSET);
+      w[i] = buf_load16_stream(prs, in ? off : OOB_OFFSET);
     }
   };
   auto issue_x = [&](int n, u32x4 (&x)[4]) {

@@ -89,7 +89,7 @@ skinny_kernel(const GemmArgs a) {
       const int row = 4 * i + (lane >> 4);
       const int lc = pc ^ (row & 7);
       const bool in = (k0 + lc * 8) < a.k;
-      wreg[i] = buf_load16(prs, in ? woff[i] + kb : OOB_OFFSET);
+      wreg[i] = buf_load16_stream(prs, in ? woff[i] + kb : OOB_OFFSET);
     }
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq)
