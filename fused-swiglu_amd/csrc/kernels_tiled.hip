@@ -497,14 +497,16 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
   store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
 }
 
-// ---- four-stage direct-to-LDS variant ------------------------------------------------------------------------
-// K tiles of 32 elements in a ring of four LDS stages: the DMA of tile kt+3 is issued while tile kt is being
-// multiplied, so a copy has three iterations (~3000 MFMA cycles) to land instead of one. That covers L2 misses
-// (Infinity Cache / HBM latency), which the two-stage kernels above expose at every barrier.
+// ---- ring-of-stages direct-to-LDS variant --------------------------------------------------------------------
+// K tiles of 32 elements in a ring of NS (4 or 5) LDS stages: the DMA of tile kt+NS-1 is issued while tile kt is
+// being multiplied, so a copy has NS-1 iterations (~1000 MFMA cycles each) to land instead of one. That covers L2
+// misses (Infinity Cache / HBM latency), which the two-stage kernels above expose at every barrier, and it keeps
+// (NS-1) stages of bytes in flight per CU: the L2 -> LDS stream of these kernels is latency-bound, so its rate
+// follows the bytes in flight. Five stages of a 256x256 tile are the whole 160 KB of LDS.
 // LDS rows are 64 bytes (4 chunks of 16 B); chunk c of row r sits at position c ^ ((r >> 2) & 3): 16 consecutive
 // rows at one logical chunk then cover the 64 banks once. The barrier waits for this wave's copy of tile kt+1
-// only (vmcnt leaves the two younger tiles in flight), hence the hand-written s_waitcnt.
-template <class E, bool GATED, bool KTAIL, int WP, int WQ, int FP, int FQ>
+// only (vmcnt leaves the younger tiles in flight), hence the hand-written s_waitcnt.
+template <class E, bool GATED, bool KTAIL, int NS, int WP, int WQ, int FP, int FQ>
 __global__ void __launch_bounds__(WP* WQ * 64)
 tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
   constexpr int NT = WP * WQ * 64;
@@ -519,13 +521,16 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
   constexpr int STAGE = (BP + BQ) * ROWB;
   static_assert(BP % RSTEP == 0 && BQ % RSTEP == 0 && RSTEP % 16 == 0, "copy mapping");
   static_assert(!GATED || (FP % 2 == 0), "gated kernel pairs fragments");
-  static_assert(4 * STAGE <= 160 * 1024, "LDS budget of a gfx950 CU");
-  static_assert(2 * NL <= 63, "vmcnt is a 6-bit counter");
+  static_assert(NS == 4 || NS == 5, "ring length");
+  static_assert(NS * STAGE <= 160 * 1024, "LDS budget of a gfx950 CU");
 
+  // one array per stage: the compiler tracks outstanding LDS DMA per array
   __shared__ __align__(1024) unsigned char ring0[STAGE];
   __shared__ __align__(1024) unsigned char ring1[STAGE];
   __shared__ __align__(1024) unsigned char ring2[STAGE];
   __shared__ __align__(1024) unsigned char ring3[STAGE];
+  __shared__ __align__(1024) unsigned char ring4[NS > 4 ? STAGE : 1024];
+  unsigned char* const ring[5] = {ring0, ring1, ring2, ring3, ring4};
 
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -629,9 +634,9 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
   using CB = std::integral_constant<int, DA + DB>;
   using CN = std::integral_constant<int, NL>;
   // s_waitcnt vmcnt(VM) lgkmcnt(0): this wave's copy of the next tile has landed (everything younger stays in
-  // flight: the tile after it and parts A and B of the one after that) and its own LDS reads are complete; then
-  // the workgroup barrier publishes every wave's part.
-  constexpr int VM = NL + DA + DB;
+  // flight: the NS-3 tiles after it and parts A and B of the one after those) and its own LDS reads are complete;
+  // then the workgroup barrier publishes every wave's part.
+  constexpr int VM = (NS - 3) * NL + DA + DB;
   static_assert(VM <= 63, "vmcnt is a 6-bit counter");
   constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
   auto ring_barrier = [&]() {
@@ -641,7 +646,7 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
   // One K tile: `cur` holds tile kt with its step-0 fragments already in pf[0]/qf[0]; `nxt` holds (or is about
   // to hold) tile kt+1; `fill` is the stage every wave finished reading before the previous barrier.
   auto iteration = [&](unsigned char* cur, unsigned char* nxt, unsigned char* fill, int kt) {
-    dma(fill, kt + 3, C0{}, CA{});
+    dma(fill, kt + NS - 1, C0{}, CA{});
     f_read(1, cur, 1);
     mma(0, 0, FP);
     if constexpr (FP == 4 && FQ == 4 && DA == 4) {
@@ -661,7 +666,7 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
     }
-    dma(fill, kt + 3, CA{}, CB{});
+    dma(fill, kt + NS - 1, CA{}, CB{});
     mma(1, 0, HF);
 #pragma unroll
     for (int i = 0; i < DB; ++i) {
@@ -670,7 +675,7 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
     }
     ring_barrier();
     f_read(0, nxt, 0);
-    dma(fill, kt + 3, CB{}, CN{});
+    dma(fill, kt + NS - 1, CB{}, CN{});
     mma(1, HF, FP);
     constexpr int MC = (FP - HF) * FQ;  // MFMAs after the barrier
 #pragma unroll
@@ -684,23 +689,26 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
     }
   };
 
+  static_assert((NS - 2) * NL <= 63, "vmcnt is a 6-bit counter");
   if (nkt > 0) {
-    dma_all(ring0, 0);
-    dma_all(ring1, 1);
-    dma_all(ring2, 2);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NL) : "memory");  // tile 0 landed, tiles 1 and 2 pending
+#pragma unroll
+    for (int j = 0; j < NS - 1; ++j) dma_all(ring[j], j);
+    // tile 0 landed, tiles 1 .. NS-2 pending
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NS - 2) * NL) : "memory");
     f_read(0, ring0, 0);
   }
   int kt = 0;
-  for (; kt + 3 < nkt; kt += 4) {
-    iteration(ring0, ring1, ring3, kt);
-    iteration(ring1, ring2, ring0, kt + 1);
-    iteration(ring2, ring3, ring1, kt + 2);
-    iteration(ring3, ring0, ring2, kt + 3);
+  for (; kt + NS - 1 < nkt; kt += NS) {
+#pragma unroll
+    for (int j = 0; j < NS; ++j) iteration(ring[j], ring[(j + 1) % NS], ring[(j + NS - 1) % NS], kt + j);
   }
-  if (kt < nkt) iteration(ring0, ring1, ring3, kt++);
-  if (kt < nkt) iteration(ring1, ring2, ring0, kt++);
-  if (kt < nkt) iteration(ring2, ring3, ring1, kt++);
+#pragma unroll
+  for (int j = 0; j < NS - 1; ++j) {
+    if (kt < nkt) {
+      iteration(ring[j], ring[(j + 1) % NS], ring[(j + NS - 1) % NS], kt);
+      ++kt;
+    }
+  }
 
   store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
 }
@@ -722,6 +730,7 @@ const TiledVariant kVariants[] = {
     {"ring8w_256x256_a", 256, 256, 512},  // 8 waves (2 per SIMD), wave tile 128 x 64
     {"ring8w_256x256_b", 256, 256, 512},  // 8 waves, wave tile 64 x 128
     {"dma8w_256x256", 256, 256, 512},
+    {"ring5_256x256", 256, 256, 256},  // five-stage ring: all 160 KB of LDS, four K tiles in flight
 };
 
 int g_raster_group = 0;  // 0 = per-launch default
@@ -757,17 +766,17 @@ hipError_t launch_dma(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
+template <class E, bool GATED, int NS, int WP, int WQ, int FP, int FQ>
 hipError_t launch_ring(const GemmArgs& a, hipStream_t stream) {
   constexpr int BP = WP * FP * 32, BQ = WQ * FQ * 32;
   const int tiles_p = (a.np + BP - 1) / BP;
   const int tiles_q = (a.nq + BQ - 1) / BQ;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
   if (a.k % 32 == 0) {
-    hipLaunchKernelGGL((tiled_ring_kernel<E, GATED, false, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
+    hipLaunchKernelGGL((tiled_ring_kernel<E, GATED, false, NS, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
                        dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, raster_group(GATED));
   } else {
-    hipLaunchKernelGGL((tiled_ring_kernel<E, GATED, true, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
+    hipLaunchKernelGGL((tiled_ring_kernel<E, GATED, true, NS, WP, WQ, FP, FQ>), dim3((unsigned)(tiles_p * tiles_q)),
                        dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, raster_group(GATED));
   }
   return hipGetLastError();
@@ -784,11 +793,12 @@ hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
     case 5: return launch_dma<E, GATED, 2, 2, 4, 4>(a, stream);
     case 6: return launch_dma<E, GATED, 2, 2, 4, 2>(a, stream);
     case 7: return launch_dma<E, GATED, 2, 2, 2, 2>(a, stream);
-    case 8: return launch_ring<E, GATED, 2, 2, 4, 4>(a, stream);
-    case 9: return launch_ring<E, GATED, 2, 2, 4, 2>(a, stream);
-    case 10: return launch_ring<E, GATED, 2, 4, 4, 2>(a, stream);
-    case 11: return launch_ring<E, GATED, 4, 2, 2, 4>(a, stream);
+    case 8: return launch_ring<E, GATED, 4, 2, 2, 4, 4>(a, stream);
+    case 9: return launch_ring<E, GATED, 4, 2, 2, 4, 2>(a, stream);
+    case 10: return launch_ring<E, GATED, 4, 2, 4, 4, 2>(a, stream);
+    case 11: return launch_ring<E, GATED, 4, 4, 2, 2, 4>(a, stream);
     case 12: return launch_dma<E, GATED, 2, 4, 4, 2>(a, stream);
+    case 13: return launch_ring<E, GATED, 5, 2, 2, 4, 4>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
