@@ -204,7 +204,9 @@ hipError_t launch_skinny_mq(int mq, int nw, const GemmArgs& a, hipStream_t strea
 SkinnyPlan skinny_plan(bool gated, int np, int nq, int k) {
   const int R = gated ? 32 : 16;
   const int tiles = (np + R - 1) / R;
-  // measured on the M=16 down projection (256 tiles): 8 waves 25.8 us, 16 waves 27.2 us, 4 waves 28.4 us
+  // measured on the M=16 down projection (256 tiles): 8 waves 25.8 us, 16 waves 27.2 us, 4 waves 28.4 us.
+  // A register ring that keeps 2, 3, 4 or 6 steps of weight loads in flight per wave measured slower than the
+  // one-step prefetch (27.5, 28.2, 29.2, 30.8 us): bytes in flight are not what limits this kernel.
   int nw = tiles <= 128 ? 16 : (tiles <= 640 ? 8 : 4);
   if (nq > 16 && nw > 8) nw = 8;
   const int nsteps = (k + 127) / 128;
