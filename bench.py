@@ -29,8 +29,9 @@ sys.path.insert(0, os.path.join(ROOT, "fused-swiglu_amd"))
 MFMA_PEAK_TFLOPS = 2516.6  # MI355X dense bf16/fp16: 256 CU x 2.4 GHz x 4096 flop/clk/CU
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # L2<->fabric bytes per launch of the dominant kernel, from separate `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
-# runs scaled by a 1 GiB copy kernel (profiles/tiled_prefill_C3_hbm_traffic_pmc.md); not measurable in-process.
-MEASURED_TRAFFIC_BYTES = {"C3": 2753080 * 1024 + 229388 * 1024}
+# runs scaled by a 1 GiB copy kernel (profiles/tiled_prefill_C3_hbm_traffic_pmc.md, skinny_decode_C4_kernel_trace.md);
+# not measurable in-process. C3: the gate/up kernel; C4: both decode kernels together.
+MEASURED_TRAFFIC_BYTES = {"C3": 2753304 * 1024 + 229390 * 1024, "C4": (230468 + 118324 + 448 + 128) * 1024}
 
 
 def parse():
@@ -168,7 +169,8 @@ def main():
         all_bytes = fsw_weights.hbm_bytes(M, d, ff)
         roofline = {"bound": "hbm", "kernel": "skinny_kernel gate/up + down (whole forward, two launches)",
                     "achieved": round(all_bytes / (gu_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(all_bytes / (gu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                    "frac": round(all_bytes / (gu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "algorithmic_bytes": all_bytes,
                     "avg_kernel_ms": round(gu_ms, 5)}
     else:
         roofline = {"bound": "mfma", "kernel": capi.variant_name(0, 0, M, 2 * ff, d) + " (gate/up)",
