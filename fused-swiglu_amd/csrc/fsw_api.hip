@@ -13,6 +13,7 @@ thread_local int g_last_hip_error = 0;
 int g_forced_variant[2] = {-1, -1};  // family 0 = gate/up, 1 = down
 
 constexpr int VARIANT_SKINNY = 100;          // id of the weight-streaming kernel in fsw_set_variant
+constexpr int VARIANT_DECODE_STREAM = 102;   // M <= 16: the streaming kernel of kernels_decode.hip, one phase per launch
 constexpr int VARIANT_DECODE_FUSED = 101;    // fsw_mlp only: single-launch decode forward (family 0)
 constexpr int64_t MAX_DIM = 1LL << 30;       // every size is cast to int inside the kernels
 constexpr int64_t MAX_LD = 1LL << 21;        // keeps tile-relative byte offsets below 2^31
@@ -52,10 +53,22 @@ int pick_tiled(int family, int64_t m, int64_t np) {
 
 int resolve_variant(int family, int64_t m, int64_t np) {
   const int forced = g_forced_variant[family];
-  if (forced == VARIANT_DECODE_FUSED) return m <= 64 ? VARIANT_SKINNY : pick_tiled(family, m, np);
+  if (forced == VARIANT_DECODE_FUSED || forced == VARIANT_DECODE_STREAM) return m <= 64 ? VARIANT_SKINNY : pick_tiled(family, m, np);
   if (forced >= 0 && !(forced == VARIANT_SKINNY && m > 64)) return forced;
   if (m <= 64) return VARIANT_SKINNY;  // decode and small batches: weight streaming, HBM bound
   return pick_tiled(family, m, np);
+}
+
+// M <= 16 with big weight matrices runs on the persistent streaming kernel of kernels_decode.hip (one phase per
+// launch) unless the caller forces the skinny kernel. Measured whole forwards at M = 16, skinny vs streaming:
+// 8192 x 28672: 260 vs 234 us; 5120 x 13824: 94.8 vs 90.0; 4096 x 14336: 63.8 vs 63.4; 4096 x 11008: 50.0 vs 54.5;
+// 2048 x 8192: 26.9 vs 31.6 (and 55.6 vs 59.1 for M = 1 at 4096 x 14336): the streaming kernel needs enough tiles
+// per CU to balance and to amortise its single reduction. K == 0 stays with the skinny kernel, which writes the
+// all-zero result.
+bool decode_stream_wanted(int family, int64_t m, int64_t rows, int64_t k) {
+  if (m > 16 || k <= 0 || g_forced_variant[family] == VARIANT_SKINNY) return false;
+  if (g_forced_variant[family] == VARIANT_DECODE_STREAM) return true;
+  return rows * k >= (family == 0 ? (int64_t)1 << 27 : (int64_t)1 << 26);  // = d * ff >= 2^26 for either projection
 }
 
 int finish(hipError_t e) {
@@ -96,7 +109,8 @@ int fsw_set_variant(int family, int variant) {
     return FSW_OK;
   }
   if (family < 0 || family > 1) return FSW_E_VARIANT;
-  if (variant >= 0 && variant != VARIANT_SKINNY && !(family == 0 && variant == VARIANT_DECODE_FUSED) &&
+  if (variant >= 0 && variant != VARIANT_SKINNY && variant != VARIANT_DECODE_STREAM &&
+      !(family == 0 && variant == VARIANT_DECODE_FUSED) &&
       variant >= fsw::tiled_variant_count())
     return FSW_E_VARIANT;
   g_forced_variant[family] = variant < 0 ? -1 : variant;
@@ -108,7 +122,7 @@ const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, i
   (void)K_or_FF;
   if (family < 0 || family > 1) return "invalid";
   const int v = resolve_variant(family, M, N_or_D);
-  if (v == VARIANT_SKINNY) return "skinny";
+  if (v == VARIANT_SKINNY) return decode_stream_wanted(family, M, N_or_D, K_or_FF) ? "decode_stream" : "skinny";
   return fsw::tiled_variant(v).name;
 }
 
@@ -162,7 +176,22 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
   a.nq = (int)M;
   a.k = (int)K;
   const int v = resolve_variant(0, M, N);
-  if (v == VARIANT_SKINNY) return finish(fsw::launch_skinny(dtype, true, a, nullptr, (hipStream_t)stream));
+  if (v == VARIANT_SKINNY) {
+    if (decode_stream_wanted(0, M, N, K)) {  // at most 16 rows: one 8-wave workgroup per CU, X held in registers
+      fsw::DecodeArgs da = {};
+      da.X = X;
+      da.W13 = W13;
+      da.H = H;
+      da.ldx = ldx;
+      da.ldw13 = ldw;
+      da.ldh = ldh;
+      da.nq = (int)M;
+      da.d = (int)K;
+      da.ff = (int)(N / 2);
+      if (fsw::decode_mlp_supported(da, 1)) return finish(fsw::launch_decode_mlp(dtype, da, (hipStream_t)stream, 1));
+    }
+    return finish(fsw::launch_skinny(dtype, true, a, nullptr, (hipStream_t)stream));
+  }
   return finish(fsw::launch_tiled(v, dtype, true, a, (hipStream_t)stream));
 }
 
@@ -193,7 +222,22 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
   a.nq = (int)M;
   a.k = (int)FF;
   const int v = resolve_variant(1, M, D);
-  if (v == VARIANT_SKINNY) return finish(fsw::launch_skinny(dtype, false, a, workspace, (hipStream_t)stream));
+  if (v == VARIANT_SKINNY) {
+    if (decode_stream_wanted(1, M, D, FF)) {
+      fsw::DecodeArgs da = {};
+      da.W2 = W2;
+      da.H = const_cast<void*>(H);
+      da.Y = Y;
+      da.ldw2 = ldw2;
+      da.ldy = ldy;
+      da.ldh = ldh;
+      da.nq = (int)M;
+      da.d = (int)D;
+      da.ff = (int)FF;
+      if (fsw::decode_mlp_supported(da, 2)) return finish(fsw::launch_decode_mlp(dtype, da, (hipStream_t)stream, 2));
+    }
+    return finish(fsw::launch_skinny(dtype, false, a, workspace, (hipStream_t)stream));
+  }
   if (need > 0 && g_forced_variant[1] < 0) {  // few output tiles, deep K: split K across workgroups
     if (!aligned16(workspace)) return FSW_E_ALIGN;
     const fsw::SplitPlan plan = fsw::tiled_split_plan((int)D, (int)M, (int)FF);
@@ -242,10 +286,11 @@ int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t 
     da.ldw13 = ldw13;
     da.ldw2 = ldw2;
     da.ldy = ldy;
+    da.ldh = FF;
     da.nq = (int)M;
     da.d = (int)D;
     da.ff = (int)FF;
-    if (fsw::decode_mlp_supported(da)) {
+    if (fsw::decode_mlp_supported(da, 3)) {
       const int drc = check_device();
       if (drc != FSW_OK) return drc;
       return finish(fsw::launch_decode_mlp(dtype, da, (hipStream_t)stream));

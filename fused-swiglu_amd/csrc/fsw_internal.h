@@ -62,10 +62,11 @@ struct DecodeArgs {
   const void* W2;
   void* H;
   void* Y;
-  long long ldx, ldw13, ldw2, ldy;  // elements
+  long long ldx, ldw13, ldw2, ldy, ldh;  // elements
   int nq, d, ff;
 };
-bool decode_mlp_supported(const DecodeArgs& a);
-hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream);
+bool decode_mlp_supported(const DecodeArgs& a, int phases = 3);
+// phases: 1 = gate/up only, 2 = down only (H already written), 3 = both in one launch
+hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream, int phases = 3);
 
 }  // namespace fsw

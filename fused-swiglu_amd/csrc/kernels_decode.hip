@@ -1,224 +1,369 @@
 // Single-launch decode forward for at most 16 activation rows on gfx950: gate/up projection, a device-wide
-// barrier, and the down projection in ONE persistent kernel (one 16-wave workgroup per CU).
+// barrier, and the down projection in ONE persistent kernel (one 8-wave workgroup per CU, up to 256 VGPRs per lane).
 //
-// Why: at M = 16 the forward moves 353 MB of weights once; two back-to-back launches leave the GPU idle for
-// ~6 us between them and each pays its own ramp-up and tail, which is 15-20 % of a ~60 us budget.
+// Why: at M = 16 the forward moves 353 MB of weights once; two back-to-back launches each pay a ramp-up and a
+// tail, and the second cannot start fetching W2 before the first has drained. Here every wave has its first
+// W2 steps in flight while the workgroups meet at the barrier, so the HBM stream does not stop between the
+// projections.
 //
-// Work split. Phase 1 walks tiles of 16 consecutive W13 rows (= 8 output features: even rows are "up", odd rows
-// "gate", swiglu.cu:380-381), phase 2 tiles of 16 W2 rows; tile t belongs to workgroup t mod (number of
-// workgroups). Inside a workgroup the 16 waves split K: wave w owns the same K slice of every tile, so its stream
-// of 4 KB steps (16 rows x 256 B, 16 lanes per row, 16 B per lane) runs across tile boundaries with two steps in
-// flight in registers. A step passes through the wave's private LDS slab (transpose to MFMA operand order, no
-// barrier) and feeds v_mfma_f32_16x16x32 with weight rows as the A operand and activation rows (from L2) as the
-// B operand. With the natural row order, accumulator registers 0/1 and 2/3 of a lane are up/gate of the same
-// feature: gating is per-lane fp32 math. Per tile the 16 partial accumulators are summed through LDS.
+// Work split. A workgroup owns a contiguous run of row tiles: in phase 1 tiles of 16 consecutive W13 rows (= 8
+// output features: even rows are "up", odd rows "gate", swiglu.cu:380-381), in phase 2 tiles of 16 W2 rows. Its
+// 8 waves split K: wave w owns the same K slice of every tile of the workgroup.
+//   Phase 1: a wave keeps the activations of its K slice in registers (four 128-element steps at a time) and
+//   streams the weight steps of up to 8 tiles past them into 8 accumulators (four steps in flight), so X is read
+//   once per wave, not once per tile, and the 8 partial sums of all tiles are reduced through LDS once at the end.
+//   Phase 2: one accumulator per tile, a register ring of 4 weight steps in flight (filled while waiting at the
+//   barrier) and the matching H fragments (loaded after the barrier).
+// A weight step is 16 rows x 256 B (16 lanes per row, 16 B per lane, non-temporal); it passes through the wave's
+// private LDS slab (transpose to MFMA operand order, no barrier) and feeds v_mfma_f32_16x16x32 with weight rows
+// as the A operand and activation rows as the B operand. With the natural W13 row order, accumulator registers
+// 0/1 and 2/3 of a lane are up/gate of the same feature: gating is per-lane fp32 math.
+// Loads past a wave's range are issued with an out-of-range offset (zero data, no memory traffic): the loops have
+// no branch around a load, so the compiler counts the loads in flight exactly.
+//
+// Visibility of H across the eight XCD-private L2s without cache-wide write-back or invalidate: phase 1 stores H
+// as relaxed agent-scope atomics (write-through to memory) and waits for their acknowledgement before arriving
+// at the barrier; no L2 holds a copy of H's lines at that point (the dispatch invalidated the L2s and nothing in
+// this kernel reads H before the barrier), so the plain loads of phase 2 miss and fetch the written data.
 //
 // Device-wide barrier: arrive/depart counters in a file-scope __device__ array (zero at module load, restored to
-// zero by the last workgroup to depart); the host hands concurrent launches different slots. Release/acquire at
-// agent scope write back and invalidate the XCD-private L2s so that H written in phase 1 is read correctly by
-// other XCDs in phase 2. The spin is bounded: if the workgroups are not all resident (someone else holds CUs)
-// the kernel gives up, raises a flag the host checks on the next call, and exits instead of hanging.
+// zero by the last workgroup to depart); the host hands concurrent launches different slots. The spin is bounded:
+// if the workgroups are not all resident (someone else holds CUs) the kernel gives up, sets the slot's `failed`
+// word (left set, for diagnosis) and finishes instead of hanging.
 #include "fsw_internal.h"
 #include "fsw_device.h"
 
 namespace fsw {
 
-constexpr int DEC_NW = 16;           // waves per workgroup
+constexpr int DEC_NW = 8;            // waves per workgroup
+constexpr int DEC_XS = 4;            // phase 1: K steps whose activations a wave holds at once = weight steps in flight
+constexpr int DEC_TG = 8;            // phase 1: tiles (accumulators) per pass
+constexpr int DEC_PF2 = 4;           // phase 2: weight steps in flight per wave
+#ifndef DEC_POLL_SLEEP
+#define DEC_POLL_SLEEP 8
+#endif
+#ifndef DEC_FILL_LATE
+#define DEC_FILL_LATE 0
+#endif
 constexpr int DEC_SLOTS = 64;        // barrier slots for concurrent launches
 constexpr unsigned DEC_SPIN_LIMIT = 1u << 18;  // ~0.3 s of polling
 static __device__ unsigned g_dec_barrier[DEC_SLOTS * 4];  // per slot: arrive, depart, failed, pad
 
-template <class E, bool GATED>
-__device__ __forceinline__ void decode_phase(const void* __restrict__ P, long long ldp, int np,
-                                             const void* __restrict__ Q, long long ldq, int nq, int k,
-                                             void* __restrict__ O, long long ldo, unsigned char* slab_all,
-                                             float* part_all) {
+// phases: bit 0 = gate/up, bit 1 = down; 3 = both with the device-wide barrier in between
+template <class E>
+__global__ void __launch_bounds__(DEC_NW * 64)
+decode_mlp_kernel(const DecodeArgs a, unsigned* bar, const int phases) {
   constexpr int KS = 128;
+  // slabs of the waves first; the phase-1 reduction reuses everything, the phase-2 reduction has its own two
+  // buffers behind the slabs
+  constexpr int LDS_BYTES = (DEC_NW * DEC_TG * 1024 > 2 * DEC_NW * 4096 + 2 * DEC_NW * 1024) ? DEC_NW * DEC_TG * 1024
+                                                                                            : 2 * DEC_NW * 4096 + 2 * DEC_NW * 1024;
+  __shared__ __align__(16) unsigned char lds[LDS_BYTES];
+
   const int t = threadIdx.x;
   const int lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int r16 = lane & 15;
   const int q = lane >> 4;
-  const int wg = blockIdx.x, nwg = gridDim.x;
-
-  const int ntiles = (np + 15) >> 4;
-  const int nt_mine = wg < ntiles ? (ntiles - wg + nwg - 1) / nwg : 0;
-  const int nsteps = (k + KS - 1) / KS;
-  const int per = (nsteps + DEC_NW - 1) / DEC_NW;
-  const int s_begin = wave * per;
-  const int s_cnt = (s_begin < nsteps) ? ((s_begin + per <= nsteps) ? per : nsteps - s_begin) : 0;
-  const int nitems = nt_mine * s_cnt;
-
-  const __amdgpu_buffer_rsrc_t prs = make_rsrc(P, ((long long)(np - 1) * ldp + k) * 2);
-  const __amdgpu_buffer_rsrc_t qrs = make_rsrc(Q, ((long long)(nq - 1) * ldq + k) * 2);
-
-  unsigned char* slab = slab_all + wave * 4096;
   const int pc = lane & 15;
+  const int wg = blockIdx.x, nwg = gridDim.x;
+  unsigned char* slab = lds + wave * 4096;
   const unsigned wr = (unsigned)lane * 16u;
   unsigned rd[4];
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) rd[kk] = (unsigned)r16 * 256u + (unsigned)(((4 * kk + q) ^ r16) * 16);
-  const unsigned xoff = (unsigned)r16 * (unsigned)ldq * 2u + (unsigned)q * 16u;
-  const unsigned row_bytes = (unsigned)ldp * 2u;
 
-  u32x4 w0[4], w1[4], x0[4], x1[4];
-  // loads of flattened item n (tile n / s_cnt, step s_begin + n % s_cnt): weights into w, activations into x
-  // Items at or beyond nitems are issued too, with every offset redirected out of range (they read zeros and
-  // touch no memory): the loop body then has no branch around a load, which lets the compiler count the loads
-  // in flight exactly instead of waiting for all of them at every control-flow join.
-  auto issue_w = [&](int n, u32x4 (&w)[4]) {
-    const bool live = n < nitems;
-    const int ti = n / s_cnt;
-    const int step = s_begin + (n - ti * s_cnt);
-    const int p0 = (wg + ti * nwg) << 4;
-    const int k0 = step * KS;
+  // one weight step: rows row0 .. row0+15, K elements k0 .. k0+127; slab chunk position pc of row `row` holds
+  // logical chunk pc ^ row (16 rows x 16 chunks). Per-lane parts of the address are loop constants (wl); the
+  // tile's row offset is added per load, the K offset goes into the scalar offset. Validity never depends on
+  // the scalar offset: rows past the matrix and dead items get an out-of-range vector offset, the K tail a
+  // per-lane predicate.
+  int lc8[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) lc8[i] = (pc ^ (4 * i + (lane >> 4))) * 8;
+  auto lane_offsets = [&](unsigned row_bytes, unsigned (&wl)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wl[i] = (unsigned)(4 * i + (lane >> 4)) * row_bytes + (unsigned)lc8[i] * 2u;
+  };
+  auto load_w = [&](__amdgpu_buffer_rsrc_t rs, const unsigned (&wl)[4], unsigned row_bytes, int row0, int k0, int kdim,
+                    bool live, u32x4 (&w)[4]) {
+    const unsigned rowpart = (unsigned)row0 * row_bytes;
+    const int krem = live ? kdim - k0 : 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int row = 4 * i + (lane >> 4);
-      const int lc = pc ^ row;  // slab chunk position pc of row `row` holds logical chunk pc ^ row (16 rows x 16 chunks)
-      const bool in = live && (k0 + lc * 8) < k;
-      const unsigned off = (unsigned)(p0 + row) * row_bytes + (unsigned)(k0 + lc * 8) * 2u;
-      w[i] = buf_load16_stream(prs, in ? off : OOB_OFFSET);
+      const unsigned voff = lc8[i] < krem ? wl[i] + rowpart : OOB_OFFSET;
+      w[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)voff, k0 * 2, 2);  // non-temporal: read exactly once
     }
   };
-  auto issue_x = [&](int n, u32x4 (&x)[4]) {
-    const bool live = n < nitems;
-    const int ti = n / s_cnt;
-    const int k0 = (s_begin + (n - ti * s_cnt)) * KS;
+  // activation fragments of one step: lane -> row r16, K chunk q of each 32-element sub-step
+  auto load_x = [&](__amdgpu_buffer_rsrc_t rs, unsigned xl, int k0, int kdim, bool live, u32x4 (&x)[4]) {
+    const int krem = live ? kdim - k0 : 0;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      const bool in = live && (k0 + kk * 32 + q * 8) < k;
-      x[kk] = buf_load16(qrs, in ? xoff + (unsigned)(k0 + kk * 32) * 2u : OOB_OFFSET);
+      const unsigned voff = (kk * 32 + q * 8) < krem ? xl : OOB_OFFSET;
+      x[kk] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)voff, k0 * 2 + kk * 64, 0);
     }
   };
+  auto to_slab = [&](u32x4 (&w)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *(u32x4*)(slab + wr + i * 1024) = w[i];
+  };
+  // workgroup barrier that orders LDS only: __syncthreads() would also wait for the weight loads in flight
+  auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  int tiles_done = 0;
-  // sum of the 16 partial accumulators of one tile, epilogue, store (wave 0 only, others go on streaming)
-  auto finalize = [&](int ti) {
-    float* part = part_all + (ti & 1) * (DEC_NW * 256);
-    *(f32x4*)(part + ((wave * 64 + lane) << 2)) = acc;
-    acc = f32x4{0.f, 0.f, 0.f, 0.f};
-    // LDS-only barrier: __syncthreads() would also wait for the weight loads in flight (vmcnt(0)) and drain
-    // the stream at every tile boundary
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    if (wave == 0) {
-      f32x4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-      for (int w = 0; w < DEC_NW; ++w) {
-        const f32x4 v = *(const f32x4*)(part + ((w * 64 + lane) << 2));
-        s[0] += v[0];
-        s[1] += v[1];
-        s[2] += v[2];
-        s[3] += v[3];
+  // ---------------------------------------------------------------- phase 1: H = (X Wu^T) * silu(X Wg^T)
+  if (phases & 1) {
+    const int np = 2 * a.ff, kdim = a.d;
+    const int ntile = (np + 15) >> 4;
+    const int tpw = (ntile + nwg - 1) / nwg;
+    const int tile0 = wg * tpw;
+    const int nsteps = (kdim + KS - 1) / KS;
+    const int per = (nsteps + DEC_NW - 1) / DEC_NW;
+    const int s_begin = wave * per;
+    const __amdgpu_buffer_rsrc_t prs = make_rsrc(a.W13, ((long long)(np - 1) * a.ldw13 + kdim) * 2);
+    const __amdgpu_buffer_rsrc_t qrs = make_rsrc(a.X, ((long long)(a.nq - 1) * a.ldx + kdim) * 2);
+    const unsigned row_bytes = (unsigned)a.ldw13 * 2u;
+    const unsigned xoff = (unsigned)r16 * (unsigned)a.ldx * 2u + (unsigned)q * 16u;
+    unsigned wl[4];
+    lane_offsets(row_bytes, wl);
+    float* red = (float*)lds;  // [wave][tile][lane][4]
+
+    for (int g0 = 0; g0 < tpw; g0 += DEC_TG) {
+      f32x4 acc[DEC_TG];
+#pragma unroll
+      for (int i = 0; i < DEC_TG; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int kb = 0; kb < per; kb += DEC_XS) {
+        u32x4 x[DEC_XS][4];
+#pragma unroll
+        for (int s = 0; s < DEC_XS; ++s) load_x(qrs, xoff, (s_begin + kb + s) * KS, kdim, kb + s < per, x[s]);
+        // items: tile-major, step-minor; item idx uses ring slot idx % DEC_XS (= its step) and accumulator
+        // idx / DEC_XS
+        u32x4 w[DEC_XS][4];
+        auto item_load = [&](int idx, u32x4 (&dst)[4]) {
+          const int ti = idx / DEC_XS, s = idx % DEC_XS;
+          const bool live = (g0 + ti < tpw) && (tile0 + g0 + ti < ntile) && (kb + s < per);
+          load_w(prs, wl, row_bytes, (tile0 + g0 + ti) << 4, (s_begin + kb + s) * KS, kdim, live, dst);
+        };
+#pragma unroll
+        for (int j = 0; j < DEC_XS; ++j) {
+          item_load(j, w[j]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int idx = 0; idx < DEC_XS * DEC_TG; ++idx) {
+          to_slab(w[idx % DEC_XS]);
+          if (idx + DEC_XS < DEC_XS * DEC_TG) item_load(idx + DEC_XS, w[idx % DEC_XS]);
+#pragma unroll
+          for (int kk = 0; kk < 4; ++kk) {
+            const u32x4 wf = *(const u32x4*)(slab + rd[kk]);
+            acc[idx / DEC_XS] = E::mfma16(wf, x[idx % DEC_XS][kk], acc[idx / DEC_XS]);
+          }
+          __builtin_amdgcn_sched_barrier(0);  // keep the items apart: merged, they would drain the ring
+        }
       }
-      const int p0 = (wg + ti * nwg) << 4;
-      const int m = r16;
-      if (m < nq) {
-        unsigned short* orow = (unsigned short*)O + (long long)m * ldo;
-        if (GATED) {
-          const int n = (p0 >> 1) + 2 * q;  // rows 4q, 4q+1 -> feature p0/2 + 2q; rows 4q+2, 4q+3 -> the next one
-          const int nout = np >> 1;
+      // sum of the 16 partial accumulators of every tile, gating, store
+      __syncthreads();  // every wave is done with its slab
+#pragma unroll
+      for (int i = 0; i < DEC_TG; ++i) *(f32x4*)(red + (((wave * DEC_TG + i) * 64 + lane) << 2)) = acc[i];
+      __syncthreads();
+      if (wave < DEC_TG && g0 + wave < tpw && tile0 + g0 + wave < ntile) {
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+        for (int w2 = 0; w2 < DEC_NW; ++w2) {
+          const f32x4 v = *(const f32x4*)(red + (((w2 * DEC_TG + wave) * 64 + lane) << 2));
+          s[0] += v[0];
+          s[1] += v[1];
+          s[2] += v[2];
+          s[3] += v[3];
+        }
+        const int p0 = (tile0 + g0 + wave) << 4;
+        const int n = (p0 >> 1) + 2 * q;  // rows 4q, 4q+1 -> feature p0/2 + 2q; rows 4q+2, 4q+3 -> the next one
+        const int nout = a.ff;
+        if (r16 < a.nq && n < nout) {
+          unsigned short* orow = (unsigned short*)a.H + (long long)r16 * a.ldh;
           const float h0 = s[0] * silu_f32(s[1]);
           const float h1 = s[2] * silu_f32(s[3]);
-          if (((ldo & 1) == 0) && n + 1 < nout) {
-            *(unsigned*)(orow + n) = E::pack2(h0, h1);
+          // the single-launch forward requires the 4-byte path (decode_mlp_supported): its stores are write-through
+          if (n + 1 < nout && ((a.ldh & 1) == 0) && ((((uintptr_t)a.H) & 3) == 0)) {
+            __hip_atomic_store((unsigned*)(orow + n), E::pack2(h0, h1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           } else {
-            if (n < nout) orow[n] = E::cvt1(h0);
+            orow[n] = E::cvt1(h0);
             if (n + 1 < nout) orow[n + 1] = E::cvt1(h1);
           }
-        } else {
-          const int n = p0 + 4 * q;
-          if (((ldo & 3) == 0) && ((((uintptr_t)O) & 7) == 0) && n + 3 < np) {
-            u32x2 pk = {E::pack2(s[0], s[1]), E::pack2(s[2], s[3])};
-            *(u32x2*)(orow + n) = pk;
-          } else {
+        }
+      }
+      __syncthreads();  // the reduction buffer overlays the slabs
+    }
+  }
+
+  // ---------------------------------------------------------------- phase 2 set-up and ring fill
+  const int np2 = a.d, k2 = a.ff;
+  const int ntile2 = (np2 + 15) >> 4;
+  const int tpw2 = (ntile2 + nwg - 1) / nwg;
+  const int tile0_2 = wg * tpw2;
+  const int nsteps2 = (k2 + KS - 1) / KS;
+  const int per2 = (nsteps2 + DEC_NW - 1) / DEC_NW;
+  const int per2p = (per2 + DEC_PF2 - 1) / DEC_PF2 * DEC_PF2;  // a tile's steps padded to whole ring rounds
+  const int nitems = tpw2 * per2p;  // the same for every wave of every workgroup
+  const __amdgpu_buffer_rsrc_t w2rs = make_rsrc(a.W2, ((long long)(np2 - 1) * a.ldw2 + k2) * 2);
+  const __amdgpu_buffer_rsrc_t hrs = make_rsrc(a.H, ((long long)(a.nq - 1) * a.ldh + k2) * 2);
+  const unsigned row_bytes2 = (unsigned)a.ldw2 * 2u;
+  // H steps are fetched like weight steps (16 lanes per row, whole cache lines) and transposed through a second
+  // slab: fetched in operand order (lane = row), every 16-lane pass of a load touches 16 different cache lines,
+  // 256 tag look-ups per step against 32, which cost a third of this phase.
+  unsigned hl[4];
+  lane_offsets((unsigned)a.ldh * 2u, hl);
+  unsigned char* hslab = lds + (DEC_NW + wave) * 4096;
+  unsigned wl2[4];
+  lane_offsets(row_bytes2, wl2);
+  // Both streams are consumed in item order, so each keeps a (tile, step) cursor instead of dividing the item
+  // index: next_w / next_h load the cursor's item and advance it.
+  int w_ti = 0, w_st = 0, h_ti = 0, h_st = 0;
+  auto next_w = [&](u32x4 (&dst)[4]) {
+    const bool live = (w_ti < tpw2) && (tile0_2 + w_ti < ntile2) && (w_st < per2);
+    load_w(w2rs, wl2, row_bytes2, (tile0_2 + w_ti) << 4, (w_st * DEC_NW + wave) * KS, k2, live, dst);
+    if (++w_st == per2p) {
+      w_st = 0;
+      ++w_ti;
+    }
+  };
+  auto next_h = [&](u32x4 (&dst)[4]) {
+    const int k0 = (h_st * DEC_NW + wave) * KS;
+    const int krem = ((h_ti < tpw2) && (h_st < per2)) ? k2 - k0 : 0;
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n + e < np) orow[n + e] = E::cvt1(s[e]);
+    for (int i = 0; i < 4; ++i)
+      dst[i] = __builtin_amdgcn_raw_buffer_load_b128(hrs, (int)(lc8[i] < krem ? hl[i] : OOB_OFFSET), k0 * 2, 0);
+    if (++h_st == per2p) {
+      h_st = 0;
+      ++h_ti;
+    }
+  };
+  // ---------------------------------------------------------------- device-wide barrier and ring fill
+  // Order: H stores acknowledged -> arrive -> fill the W2 ring -> wait for the others. A workgroup that finishes
+  // phase 1 early spends its wait fetching W2; a late one arrives without waiting for its own ring.
+  u32x4 w2[DEC_PF2][4];
+  if (phases == 3) {
+    __syncthreads();  // vmcnt(0): every store of H by this workgroup has been acknowledged by memory
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(bar + 0, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // Wave 0 polls the barrier, and loads return in order: with its own ring fill in flight (queued behind every
+  // other workgroup's) the poll result would arrive microseconds late, so wave 0 fills its ring after the barrier.
+  auto fill_ring = [&]() {
+#pragma unroll
+    for (int j = 0; j < DEC_PF2; ++j) {
+      next_w(w2[j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  const bool fill_late = (phases == 3) && wave == 0 && DEC_FILL_LATE;
+  if ((phases & 2) && !fill_late) fill_ring();
+  if (phases == 3) {
+    if (threadIdx.x == 0) {
+      unsigned spins = 0;
+      while (__hip_atomic_load(bar + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gridDim.x) {
+        if (++spins > DEC_SPIN_LIMIT) {  // not all workgroups are resident: give up rather than hang
+          __hip_atomic_store(bar + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(DEC_POLL_SLEEP);  // 256 pollers must not saturate the counter's channel
+      }
+      // depart: the last workgroup out restores the slot for the next launch that is handed it
+      const unsigned left = __hip_atomic_fetch_add(bar + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (left == gridDim.x - 1) {
+        __hip_atomic_store(bar + 0, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(bar + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    lds_barrier();  // no vmcnt wait: the ring stays in flight; also keeps loads of H below the barrier
+    if (fill_late) fill_ring();
+  }
+
+  // ---------------------------------------------------------------- phase 2: Y = H W2^T
+  if (phases & 2) {
+    float* part_all = (float*)(lds + 2 * DEC_NW * 4096);  // two buffers of [wave][lane][4], by tile parity
+    // H fragments ride the same ring distance as the weights and are issued before them: loads return in
+    // order, so a younger, shorter H ring would make every step wait for the weight loads issued ahead of it
+    u32x4 xh[DEC_PF2][4];
+#pragma unroll
+    for (int j = 0; j < DEC_PF2; ++j) {
+      next_h(xh[j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    f32x4 acc2 = {0.f, 0.f, 0.f, 0.f};
+    int st_done = 0, ti_done = 0;
+#pragma nounroll
+    for (int i = 0; i < nitems; i += DEC_PF2) {
+#pragma unroll
+      for (int j = 0; j < DEC_PF2; ++j) {
+        to_slab(w2[j]);
+#pragma unroll
+        for (int i2 = 0; i2 < 4; ++i2) *(u32x4*)(hslab + wr + i2 * 1024) = xh[j][i2];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const u32x4 wf = *(const u32x4*)(slab + rd[kk]);
+          const u32x4 hf = *(const u32x4*)(hslab + rd[kk]);
+          acc2 = E::mfma16(wf, hf, acc2);
+        }
+        next_h(xh[j]);
+        next_w(w2[j]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      st_done += DEC_PF2;
+      if (st_done == per2p) {  // a tile is complete (uniform over the workgroup)
+        st_done = 0;
+        const int tile = tile0_2 + ti_done;
+        float* part = part_all + (ti_done & 1) * (DEC_NW * 256);
+        ++ti_done;
+        *(f32x4*)(part + ((wave * 64 + lane) << 2)) = acc2;
+        acc2 = f32x4{0.f, 0.f, 0.f, 0.f};
+        lds_barrier();
+        if (wave == 0 && tile < ntile2) {
+          f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+          for (int w = 0; w < DEC_NW; ++w) {
+            const f32x4 v = *(const f32x4*)(part + ((w * 64 + lane) << 2));
+            s[0] += v[0];
+            s[1] += v[1];
+            s[2] += v[2];
+            s[3] += v[3];
+          }
+          const int n = (tile << 4) + 4 * q;
+          if (r16 < a.nq) {
+            unsigned short* orow = (unsigned short*)a.Y + (long long)r16 * a.ldy;
+            if (((a.ldy & 3) == 0) && ((((uintptr_t)a.Y) & 7) == 0) && n + 3 < np2) {
+              u32x2 pk = {E::pack2(s[0], s[1]), E::pack2(s[2], s[3])};
+              *(u32x2*)(orow + n) = pk;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (n + e < np2) orow[n + e] = E::cvt1(s[e]);
+            }
           }
         }
       }
     }
-    ++tiles_done;
-  };
-  // registers -> slab frees w for the loads two items ahead; x is free again once the MFMAs have consumed it
-  auto process = [&](int n, u32x4 (&w)[4], u32x4 (&x)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *(u32x4*)(slab + wr + i * 1024) = w[i];
-    issue_w(n + 2, w);
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const u32x4 wf = *(const u32x4*)(slab + rd[kk]);
-      acc = E::mfma16(wf, x[kk], acc);
-    }
-    issue_x(n + 2, x);
-    if (n < nitems && (n + 1) % s_cnt == 0) finalize(n / s_cnt);
-  };
-
-  if (nitems > 0) {  // s_cnt > 0 from here on
-    issue_w(0, w0);
-    issue_x(0, x0);
-    issue_w(1, w1);
-    issue_x(1, x1);
-    for (int n = 0; n < nitems; n += 2) {
-      process(n, w0, x0);
-      process(n + 1, w1, x1);  // a dead item when nitems is odd: zero operands, no reduction
-    }
   }
-  // waves without a K slice still take part in every tile's reduction barrier
-  while (tiles_done < nt_mine) finalize(tiles_done);
 }
 
-template <class E>
-__global__ void __launch_bounds__(DEC_NW * 64)
-decode_mlp_kernel(const DecodeArgs a, unsigned* bar) {
-  __shared__ __align__(16) unsigned char slab[DEC_NW * 4096];
-  __shared__ __align__(16) float part[2 * DEC_NW * 256];
-
-  decode_phase<E, true>(a.W13, a.ldw13, 2 * a.ff, a.X, a.ldx, a.nq, a.d, a.H, a.ff, slab, part);
-
-  // ---- device-wide barrier between the phases
-  __syncthreads();  // every store of H by this workgroup has been issued and acknowledged
-  if (threadIdx.x == 0) {
-    __hip_atomic_fetch_add(bar + 0, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);  // writes back this XCD's L2
-    unsigned spins = 0;
-    // relaxed polling: an acquire load would invalidate the XCD's L2 on every iteration while other
-    // workgroups are still streaming; one acquire fence after the barrier is enough
-    while (__hip_atomic_load(bar + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gridDim.x) {
-      if (++spins > DEC_SPIN_LIMIT) {  // not all workgroups are resident: give up rather than hang
-        __hip_atomic_store(bar + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(16);  // ~0.5 us between polls: 256 pollers must not load the counter's channel
-    }
-    // one acquire per workgroup: invalidates this CU's L1 and this XCD's L2 copies of lines other XCDs wrote
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    // depart: the last workgroup out restores the slot for the next launch that is handed it
-    const unsigned left = __hip_atomic_fetch_add(bar + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (left == gridDim.x - 1) {
-      __hip_atomic_store(bar + 0, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(bar + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
-  __syncthreads();
-
-  decode_phase<E, false>(a.W2, a.ldw2, a.d, a.H, a.ff, a.nq, a.ff, a.Y, a.ldy, slab, part);
-}
-
-bool decode_mlp_supported(const DecodeArgs& a) {
-  if (a.nq < 1 || a.nq > 16 || a.d < 8 || a.ff < 8) return false;
-  // one buffer descriptor spans a whole matrix: byte offsets must stay below 2^31
+bool decode_mlp_supported(const DecodeArgs& a, int phases) {
+  if (a.nq < 1 || a.nq > 16 || a.d < 8 || a.ff < 1) return false;
+  if ((phases & 2) && a.ff < 8) return false;
+  // one launch for both phases: H must take the 4-byte write-through stores everywhere
+  if (phases == 3 && ((a.ff & 1) || (a.ldh & 1) || (((uintptr_t)a.H) & 3))) return false;
+  // one buffer descriptor spans a whole matrix and a partial last tile addresses up to 15 rows past it: byte
+  // offsets must stay below 2^31
   const long long lim = 0x7fffffffLL;
-  if ((long long)2 * a.ff * a.ldw13 * 2 >= lim) return false;
-  if ((long long)a.d * a.ldw2 * 2 >= lim) return false;
+  if ((phases & 1) && ((long long)2 * a.ff + 16) * a.ldw13 * 2 >= lim) return false;
+  if ((phases & 2) && ((long long)a.d + 16) * a.ldw2 * 2 >= lim) return false;
+  if ((phases & 2) && 16 * a.ldh * 2 >= lim) return false;
   return true;
 }
 
-hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream) {
+hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream, int phases) {
   static int cu_count[64] = {0};
   static unsigned* bar_base[64] = {nullptr};
   static unsigned next_slot = 0;
+  if (phases < 1 || phases > 3) return hipErrorInvalidValue;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
@@ -235,14 +380,14 @@ hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream)
   }
   const unsigned slot = __atomic_fetch_add(&next_slot, 1u, __ATOMIC_RELAXED) % DEC_SLOTS;
   unsigned* bar = bar_base[dev] + slot * 4;
-  const int tiles1 = (2 * a.ff + 15) / 16, tiles2 = (a.d + 15) / 16;
+  const int tiles1 = (phases & 1) ? (2 * a.ff + 15) / 16 : 0, tiles2 = (phases & 2) ? (a.d + 15) / 16 : 0;
   int grid = cu_count[dev];  // one workgroup per CU: all resident at once, which the barrier relies on
   const int most = tiles1 > tiles2 ? tiles1 : tiles2;
   if (grid > most) grid = most;
   if (dtype == 0) {
-    hipLaunchKernelGGL((decode_mlp_kernel<Bf16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar);
+    hipLaunchKernelGGL((decode_mlp_kernel<Bf16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar, phases);
   } else {
-    hipLaunchKernelGGL((decode_mlp_kernel<Fp16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar);
+    hipLaunchKernelGGL((decode_mlp_kernel<Fp16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar, phases);
   }
   return hipGetLastError();
 }

@@ -140,6 +140,39 @@ def test_skinny_weight_streaming_variant(capi, M, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [1, 7, 16])
+def test_streaming_decode_variant(capi, M, dtype):
+    """The persistent streaming kernel for M <= 16, one projection per launch (variant 102; picked automatically
+    only for large d * ff): ragged d / ff, more tiles than one pass of accumulators holds (ff = 20000 at 8 features
+    per tile on few CUs is covered by d = 40: many tiles per workgroup), K slices longer than the activation
+    registers (d = 9000), odd ff with scalar stores."""
+    try:
+        capi.set_variant(0, 102)
+        capi.set_variant(1, 102)
+        for (d, ff) in [(8, 8), (136, 40), (1000, 264), (4096, 520), (256, 2056), (40, 20000), (9000, 72)]:
+            inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=41 * M + d, x_scale=0.5)
+            g = to_dev(inp)
+            assert capi.variant_name(0, 0, M, 2 * ff, d) == "decode_stream"
+            assert capi.variant_name(1, 0, M, d, ff) == "decode_stream"
+            H = capi.gateup(g["X"], g["W13"])
+            assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype,
+                                "stream H %s" % ((M, d, ff),))
+            Y = capi.down(H, g["W2"])
+            assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype,
+                                "stream Y %s" % ((M, d, ff),))
+        inp = fsw_weights.make_inputs(M, 72, 37, dtype, seed=6, x_scale=0.5)
+        H = capi.gateup(inp["X"].to(DEV), inp["W13"].to(DEV))
+        assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "stream odd ff")
+        # above 16 rows the override falls back to the dispatcher's choice
+        assert capi.variant_name(0, 0, 17, 2 * 264, 1000) == "skinny"
+    finally:
+        capi.set_variant(0, -1)
+        capi.set_variant(1, -1)
+    assert capi.variant_name(0, 0, 16, 2 * 28672, 8192) == "decode_stream"
+    assert capi.variant_name(0, 0, 16, 2 * 14336, 4096) == "skinny"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [1, 5, 16])
 def test_single_launch_decode_forward(capi, M, dtype):
     """With variant 101 fsw_mlp runs M <= 16 as one launch (gate/up, device-wide barrier, down projection); it
@@ -154,6 +187,12 @@ def test_single_launch_decode_forward(capi, M, dtype):
             Y1 = capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws)
             H1 = ws[: M * ff * 2].view(dtype).view(M, ff).clone()
             reps = [capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws) for _ in range(3)]  # barrier slots are reused
+            # other activations through the same H scratch: phase 2 must read what THIS call's phase 1 wrote,
+            # from whichever XCD wrote it, not lines an L2 kept from the previous call
+            inp_b = fsw_weights.make_inputs(M, d, ff, dtype, seed=9000 + 77 * M + d, x_scale=0.5)
+            Xb = inp_b["X"].to(DEV)
+            Yb = capi.mlp(Xb, g["W13"], g["W2"], workspace=ws)
+            Ya = capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws)
         finally:
             capi.set_variant(0, -1)
         Y2 = capi.mlp(g["X"], g["W13"], g["W2"])
@@ -166,6 +205,8 @@ def test_single_launch_decode_forward(capi, M, dtype):
         assert (Y1.float() - Y2.float()).abs().max().item() <= 2e-2
         for r in reps:
             assert torch.equal(r, Y1)
+        oracle.assert_parity(Yb, oracle.ref_mlp(inp_b["X"], inp["W13"], inp["W2"], torch.float64), "fused mlp, second input %s" % ((M, d, ff),))
+        assert torch.equal(Ya, Y1)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
