@@ -108,6 +108,18 @@ def test_variant_choice_by_regime(capi):
     assert name(0, 16, 28672, 4096) == "skinny" and name(1, 1, 4096, 14336) == "skinny"
     assert name(0, 64, 28672, 4096) == "skinny" and name(1, 33, 4096, 14336) == "skinny"
     assert name(0, 100, 28672, 4096) == "dma_128x128"
+    # at most 16 rows and d * ff >= 2^26: the persistent streaming kernel, one projection per launch
+    assert name(0, 16, 2 * 28672, 8192) == "decode_stream" and name(1, 16, 8192, 28672) == "decode_stream"
+    assert name(0, 17, 2 * 28672, 8192) == "skinny"
+    L = capi.lib()
+    try:
+        assert L.fsw_set_variant(0, 102) == capi.OK and L.fsw_set_variant(1, 100) == capi.OK
+        assert name(0, 4, 64, 32) == "decode_stream" and name(0, 17, 64, 32) == "skinny"
+        assert name(1, 16, 8192, 28672) == "skinny"          # forced weight-streaming kernel wins over the size rule
+        assert L.fsw_set_variant(1, 101) == capi.E_VARIANT   # the single-launch form is a family-0 (fsw_mlp) option
+    finally:
+        L.fsw_set_variant(0, -1)
+        L.fsw_set_variant(1, -1)
     # the down product with few output tiles and a deep K asks for split-K scratch; large or tiny M does not
     ws = capi.lib().fsw_down_workspace_bytes
     assert ws(0, 256, 4096, 14336) == 8 * 256 * 4096 * 4
