@@ -59,16 +59,15 @@ int resolve_variant(int family, int64_t m, int64_t np) {
   return pick_tiled(family, m, np);
 }
 
-// M <= 16 with big weight matrices runs on the persistent streaming kernel of kernels_decode.hip (one phase per
-// launch) unless the caller forces the skinny kernel. Measured whole forwards at M = 16, skinny vs streaming:
-// 8192 x 28672: 260 vs 234 us; 5120 x 13824: 94.8 vs 90.0; 4096 x 14336: 63.8 vs 63.4; 4096 x 11008: 50.0 vs 54.5;
-// 2048 x 8192: 26.9 vs 31.6 (and 55.6 vs 59.1 for M = 1 at 4096 x 14336): the streaming kernel needs enough tiles
-// per CU to balance and to amortise its single reduction. K == 0 stays with the skinny kernel, which writes the
-// all-zero result.
+// M <= 16 with very large weight matrices runs on the persistent streaming kernel of kernels_decode.hip (one phase
+// per launch) unless the caller forces the skinny kernel. Measured whole forwards at M = 16, skinny vs streaming:
+// 8192 x 28672: 254 vs 233 us; 5120 x 13824: 87.6 vs 90.3; 4096 x 14336: 61.1 vs 63.4; 4096 x 11008: 50.0 vs 54.5;
+// 2048 x 8192: 26.9 vs 31.6: the streaming kernel needs many tiles per CU to balance and to amortise its single
+// reduction. K == 0 stays with the skinny kernel, which writes the all-zero result.
 bool decode_stream_wanted(int family, int64_t m, int64_t rows, int64_t k) {
   if (m > 16 || k <= 0 || g_forced_variant[family] == VARIANT_SKINNY) return false;
   if (g_forced_variant[family] == VARIANT_DECODE_STREAM) return true;
-  return rows * k >= (family == 0 ? (int64_t)1 << 27 : (int64_t)1 << 26);  // = d * ff >= 2^26 for either projection
+  return rows * k >= (family == 0 ? (int64_t)1 << 28 : (int64_t)1 << 27);  // = d * ff >= 2^27 for either projection
 }
 
 int finish(hipError_t e) {

@@ -22,13 +22,19 @@
 
 namespace fsw {
 
-template <class E, bool GATED, int MQ, int NW>
+template <class E, bool GATED, int MQ, int NW, bool XSLAB>
 __global__ void __launch_bounds__(NW * 64)
 skinny_kernel(const GemmArgs a) {
   constexpr int T = GATED ? 2 : 1;   // accumulator sets (up, gate)
   constexpr int R = 16 * T;          // weight rows per tile
   constexpr int NL = R / 4;          // weight loads per lane per step
   constexpr int KS = 128;            // K elements per step
+  // Activations pass through the slab too: fetched like weights, 16 lanes per row, every 16-lane pass of a load
+  // covers two whole cache lines; fetched in operand order (lane = row) every pass touches 16 lines, 256 tag
+  // look-ups per 16-row step where 32 suffice. They go first (write, read back as fragments), then the weights
+  // reuse the same bytes: LDS serves a wave's accesses in order. Measured on whole forwards at 4096 x 14336:
+  // M = 16: 63.7 -> 61.0 us, M = 32: 85.8 -> 73.0, M = 64: 134.5 -> 98.1; with few activation rows the direct fetch
+  // touches few lines per pass anyway (M = 3: 1.3 % faster, M = 8: level), so XSLAB is off for nq <= 8.
   constexpr int SLAB = R * 256;      // bytes of one wave's transpose buffer
   static_assert(MQ * T * 1024 <= SLAB, "the reduction reuses the slabs");
   __shared__ __align__(16) unsigned char lds[NW * SLAB];
@@ -79,6 +85,15 @@ skinny_kernel(const GemmArgs a) {
 #pragma unroll
     for (int mq = 0; mq < MQ; ++mq) acc[s][mq] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // coalesced activation mapping (XSLAB): load i covers rows 4i .. 4i+3 of the 16-row block, like the weights
+  unsigned xoffc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 4 * i + (lane >> 4);
+    xoffc[i] = (unsigned)row * (unsigned)a.ldq * 2u + (unsigned)(pc ^ (row & 7)) * 16u;
+  }
+  const unsigned xblock = 16u * (unsigned)a.ldq * 2u;  // bytes between 16-row activation blocks
+
   u32x4 wreg[NL];
   u32x4 xreg[MQ][4];
   auto g_load = [&](int step) {
@@ -91,25 +106,48 @@ skinny_kernel(const GemmArgs a) {
       const bool in = (k0 + lc * 8) < a.k;
       wreg[i] = buf_load16_stream(prs, in ? woff[i] + kb : OOB_OFFSET);
     }
+    if constexpr (XSLAB) {
 #pragma unroll
-    for (int mq = 0; mq < MQ; ++mq)
+      for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const bool in = (k0 + kk * 32 + q * 8) < a.k;
-        xreg[mq][kk] = buf_load16(qrs, in ? xoff[mq] + kb + (unsigned)kk * 64u : OOB_OFFSET);
-      }
+        for (int i = 0; i < 4; ++i) {
+          const int row = 4 * i + (lane >> 4);
+          const int lc = pc ^ (row & 7);
+          const bool in = (k0 + lc * 8) < a.k;
+          xreg[mq][i] = buf_load16(qrs, in ? xoffc[i] + (unsigned)mq * xblock + kb : OOB_OFFSET);
+        }
+    } else {
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq)
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const bool in = (k0 + kk * 32 + q * 8) < a.k;
+          xreg[mq][kk] = buf_load16(qrs, in ? xoff[mq] + kb + (unsigned)kk * 64u : OOB_OFFSET);
+        }
+    }
   };
 
   if (s_begin < s_end) g_load(s_begin);
   for (int step = s_begin; step < s_end; ++step) {
     // registers -> slab (waits for this step's loads), then free the registers for the next step's loads
+    u32x4 xcur[MQ][4];
+    if constexpr (XSLAB) {
+#pragma unroll
+      for (int mq = 0; mq < MQ; ++mq) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *(u32x4*)(slab + wr + i * 1024) = xreg[mq][i];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) xcur[mq][kk] = *(const u32x4*)(slab + rd[kk]);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < NL; ++i) *(u32x4*)(slab + wr + i * 1024) = wreg[i];
-    u32x4 xcur[MQ][4];
+    if constexpr (!XSLAB) {
 #pragma unroll
-    for (int mq = 0; mq < MQ; ++mq)
+      for (int mq = 0; mq < MQ; ++mq)
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) xcur[mq][kk] = xreg[mq][kk];
+        for (int kk = 0; kk < 4; ++kk) xcur[mq][kk] = xreg[mq][kk];
+    }
     if (step + 1 < s_end) g_load(step + 1);
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
@@ -173,7 +211,13 @@ hipError_t launch_skinny_one(const GemmArgs& a, hipStream_t stream) {
   constexpr int R = GATED ? 32 : 16;
   const int tiles = (a.np + R - 1) / R;
   if (tiles <= 0) return hipSuccess;
-  hipLaunchKernelGGL((skinny_kernel<E, GATED, MQ, NW>), dim3((unsigned)tiles), dim3(NW * 64), 0, stream, a);
+  if constexpr (MQ == 1) {
+    if (a.nq <= 8) {
+      hipLaunchKernelGGL((skinny_kernel<E, GATED, MQ, NW, false>), dim3((unsigned)tiles), dim3(NW * 64), 0, stream, a);
+      return hipGetLastError();
+    }
+  }
+  hipLaunchKernelGGL((skinny_kernel<E, GATED, MQ, NW, true>), dim3((unsigned)tiles), dim3(NW * 64), 0, stream, a);
   return hipGetLastError();
 }
 

@@ -108,7 +108,7 @@ def test_variant_choice_by_regime(capi):
     assert name(0, 16, 28672, 4096) == "skinny" and name(1, 1, 4096, 14336) == "skinny"
     assert name(0, 64, 28672, 4096) == "skinny" and name(1, 33, 4096, 14336) == "skinny"
     assert name(0, 100, 28672, 4096) == "dma_128x128"
-    # at most 16 rows and d * ff >= 2^26: the persistent streaming kernel, one projection per launch
+    # at most 16 rows and d * ff >= 2^27: the persistent streaming kernel, one projection per launch
     assert name(0, 16, 2 * 28672, 8192) == "decode_stream" and name(1, 16, 8192, 28672) == "decode_stream"
     assert name(0, 17, 2 * 28672, 8192) == "skinny"
     L = capi.lib()
