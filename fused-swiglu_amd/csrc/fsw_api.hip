@@ -247,6 +247,99 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
   return finish(fsw::launch_tiled(v, dtype, false, a, (hipStream_t)stream));
 }
 
+// Large-tile regime of fsw_mlp: both projections run 256 x 256 tiles, so X is re-blocked once into the workspace
+// and H never exists row-major (the gate/up epilogue writes it blocked, the down projection reads it blocked).
+static bool blocked_regime(int64_t M, int64_t D, int64_t FF) {
+  if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[0] >= 0 || g_forced_variant[1] >= 0) return false;
+  return pick_tiled(0, M, 2 * FF) == 8 && pick_tiled(1, M, D) == 5;
+}
+
+size_t fsw_blocked_bytes(int64_t rows, int64_t k) {
+  if (rows <= 0 || k <= 0 || rows > MAX_DIM || k > MAX_DIM) return 0;
+  return (size_t)fsw::blocked_bytes(rows, k);
+}
+
+// src: row-major [rows, k], 16-byte aligned, ld and k multiples of 8; dst: fsw_blocked_bytes(rows, k) bytes
+static int block_rows_impl(int dtype, int64_t rows, int64_t k, const void* src, int64_t ld, void* dst, bool gated_order,
+                           void* stream) {
+  if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
+  if (rows < 0 || k < 0 || rows > MAX_DIM || k > MAX_DIM || (gated_order && (rows & 1))) return FSW_E_SHAPE;
+  if (rows == 0 || k == 0) return FSW_OK;
+  if (!src || !dst) return FSW_E_NULL;
+  if (ld < k) return FSW_E_LD;
+  if (ld > MAX_LD) return FSW_E_SHAPE;
+  if ((k & 7) || (ld & 7) || !aligned16(src) || !aligned16(dst)) return FSW_E_ALIGN;
+  const int drc = check_device();
+  if (drc != FSW_OK) return drc;
+  return finish(fsw::launch_block_rows(src, ld, (int)rows, (int)k, dst, gated_order, (hipStream_t)stream));
+}
+
+int fsw_block_rows(int dtype, int64_t rows, int64_t k, const void* src, int64_t ld, void* dst, void* stream) {
+  return block_rows_impl(dtype, rows, k, src, ld, dst, false, stream);
+}
+
+int fsw_prepack_w13(int dtype, int64_t N, int64_t K, const void* W13, int64_t ldw, void* dst, void* stream) {
+  return block_rows_impl(dtype, N, K, W13, ldw, dst, true, stream);
+}
+
+int fsw_prepack_w2(int dtype, int64_t D, int64_t FF, const void* W2, int64_t ldw2, void* dst, void* stream) {
+  return block_rows_impl(dtype, D, FF, W2, ldw2, dst, false, stream);
+}
+
+int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* Xb, const void* W13, int64_t ldw,
+                       int w_blocked, void* Hb, void* stream) {
+  if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
+  if (M < 0 || N < 0 || K < 0 || (N & 1) || M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return FSW_E_SHAPE;
+  if (M == 0 || N == 0) return FSW_OK;
+  if (K == 0) return FSW_E_SHAPE;  // a blocked matrix with no columns has no representation
+  if (!Xb || !W13 || !Hb) return FSW_E_NULL;
+  if (!w_blocked && ldw < K) return FSW_E_LD;
+  if (!w_blocked && ldw > MAX_LD) return FSW_E_SHAPE;
+  if ((K & 7) || (!w_blocked && (ldw & 7))) return FSW_E_ALIGN;
+  if (!aligned16(Xb) || !aligned16(W13) || !aligned16(Hb)) return FSW_E_ALIGN;
+  const int drc = check_device();
+  if (drc != FSW_OK) return drc;
+  fsw::GemmArgs a;
+  a.P = W13;
+  a.Q = Xb;
+  a.O = Hb;
+  a.ldp = ldw;
+  a.ldq = 0;
+  a.ldo = 0;
+  a.np = (int)N;
+  a.nq = (int)M;
+  a.k = (int)K;
+  a.layout = w_blocked ? 7 : 3;
+  return finish(fsw::launch_tiled_blocked(dtype, true, a, (hipStream_t)stream));
+}
+
+int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* Hb, const void* W2, int64_t ldw2,
+                     int w_blocked, void* Y, int64_t ldy, void* stream) {
+  if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
+  if (M < 0 || D < 0 || FF < 0 || M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM) return FSW_E_SHAPE;
+  if (M == 0 || D == 0) return FSW_OK;
+  if (FF == 0) return FSW_E_SHAPE;
+  if (!Hb || !W2 || !Y) return FSW_E_NULL;
+  if ((!w_blocked && ldw2 < FF) || ldy < D) return FSW_E_LD;
+  if ((!w_blocked && ldw2 > MAX_LD) || ldy > MAX_DIM) return FSW_E_SHAPE;
+  if ((FF & 7) || (!w_blocked && (ldw2 & 7)) || (((uintptr_t)Y) & 1)) return FSW_E_ALIGN;
+  if (!aligned16(Hb) || !aligned16(W2)) return FSW_E_ALIGN;
+  const int drc = check_device();
+  if (drc != FSW_OK) return drc;
+  fsw::GemmArgs a;
+  a.P = W2;
+  a.Q = Hb;
+  a.O = Y;
+  a.ldp = ldw2;
+  a.ldq = 0;
+  a.ldo = ldy;
+  a.np = (int)D;
+  a.nq = (int)M;
+  a.k = (int)FF;
+  a.layout = w_blocked ? 5 : 1;
+  return finish(fsw::launch_tiled_blocked(dtype, false, a, (hipStream_t)stream));
+}
+
 static size_t h_bytes(int64_t M, int64_t FF) {
   const size_t raw = (size_t)M * (size_t)FF * 2;
   return (raw + 255) & ~(size_t)255;
@@ -254,6 +347,7 @@ static size_t h_bytes(int64_t M, int64_t FF) {
 
 size_t fsw_mlp_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
   if (M <= 0 || D <= 0 || FF <= 0) return 0;
+  if (blocked_regime(M, D, FF)) return (size_t)fsw::blocked_bytes(M, FF) + (size_t)fsw::blocked_bytes(M, D);
   return h_bytes(M, FF) + fsw_down_workspace_bytes(dtype, M, D, FF);
 }
 
@@ -294,6 +388,15 @@ int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t 
       if (drc != FSW_OK) return drc;
       return finish(fsw::launch_decode_mlp(dtype, da, (hipStream_t)stream));
     }
+  }
+  if (blocked_regime(M, D, FF)) {  // workspace = [H blocked][X blocked]
+    unsigned char* Hb = (unsigned char*)workspace;
+    unsigned char* Xb = Hb + fsw::blocked_bytes(M, FF);
+    rc = fsw_block_rows(dtype, M, D, X, ldx, Xb, stream);
+    if (rc != FSW_OK) return rc;
+    rc = fsw_gateup_blocked(dtype, M, 2 * FF, D, Xb, W13, ldw13, 0, Hb, stream);
+    if (rc != FSW_OK) return rc;
+    return fsw_down_blocked(dtype, M, D, FF, Hb, W2, ldw2, 0, Y, ldy, stream);
   }
   rc = fsw_gateup(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF, stream);
   if (rc != FSW_OK) return rc;

@@ -20,7 +20,14 @@ struct GemmArgs {
   // store fp32 partial sums to partial[split][nq][np]; splitk_reduce() sums them and rounds once.
   int splits = 1;
   float* partial = nullptr;
+  // panel-blocked operands / output of the 256 x 256 ring kernel (launch_tiled_blocked): bit 0 = Q, bit 1 = O
+  // (gated kernel), bit 2 = P. A blocked [rows, k] matrix is ceil(rows / 256) panels of ceil(k / 32) blocks of
+  // [256 rows][64 bytes], zero padded (blocked_bytes()).
+  int layout = 0;
 };
+inline long long blocked_bytes(long long rows, long long k) {
+  return ((rows + 255) / 256) * ((k + 31) / 32) * (256 * 64);
+}
 
 // Tiled LDS/MFMA kernels (kernels_tiled.hip). `variant` indexes tiled_variant_table().
 struct TiledVariant {
@@ -32,6 +39,11 @@ void set_raster_group(int g);  // activation-row tiles per raster band; 0 restor
 int tiled_variant_count();
 const TiledVariant& tiled_variant(int variant);
 hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
+// gated: layout 3 (X blocked in, H blocked out) or 7 (+ W13 blocked); plain: layout 1 (H blocked in) or 5 (+ W2 blocked)
+hipError_t launch_tiled_blocked(int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
+// row-major [rows, k] (row stride ld elements) -> blocked; gated_order: W13's up/gate rows de-interleaved per panel
+hipError_t launch_block_rows(const void* src, long long ld, int rows, int k, void* dst, bool gated_order,
+                             hipStream_t stream);
 // Plan for the plain (down-projection) product when the output has few tiles and K is deep: which direct-to-LDS
 // tile (128 or 256 square) and how many K partitions, so that about two workgroups per CU are in flight.
 // splits == 1 means the ordinary launch path.

@@ -68,6 +68,38 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[FP][FQ], const GemmArgs
   }
 }
 
+// Gated epilogue that writes H panel-blocked for the down projection: panels of 256 activation rows, blocks of
+// 32 features, block (panel, j) = [256 rows][64 bytes] at ((panel * nblocks + j) * 256 + row) * 64. Every row of the
+// panel and every feature up to the next multiple of 32 is written: rows past nq and features past ff come from
+// out-of-range (zero) operand rows, so the padding the down projection's K loop reads is zero.
+template <class E, int WP, int WQ, int FP, int FQ>
+__device__ __forceinline__ void store_tile_blocked(f32x16 (&acc)[FP][FQ], const GemmArgs& a, int tp, int tq, int wp,
+                                                   int wq, int l32, int hi) {
+  constexpr int FO = FP / 2;
+  constexpr int BH = WP * FO;  // 32-feature blocks per tile
+  const int nblocks = (a.np / 2 + 31) >> 5;
+  unsigned char* O = (unsigned char*)a.O;
+#pragma unroll
+  for (int g = 0; g < FQ; ++g) {
+    const int row = (wq * FQ + g) * 32 + l32;
+#pragma unroll
+    for (int f = 0; f < FO; ++f) {
+      const int blk = tp * BH + wp * FO + f;
+      if (blk < nblocks) {
+        unsigned char* dst = O + (((long long)tq * nblocks + blk) * 256 + row) * 64 + hi * 8;
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = acc[f][g][i4 * 4 + e] * silu_f32(acc[f + FO][g][i4 * 4 + e]);
+          u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
+          *(u32x2*)(dst + i4 * 16) = pk;
+        }
+      }
+    }
+  }
+}
+
 // Split-K epilogue of the plain kernel: fp32 partial sums to partial[split][m][n], 16 bytes per lane.
 template <int WP, int WQ, int FP, int FQ>
 __device__ __forceinline__ void store_partial(f32x16 (&acc)[FP][FQ], const GemmArgs& a, int split, int p0, int q0,
@@ -506,7 +538,13 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
 // LDS rows are 64 bytes (4 chunks of 16 B); chunk c of row r sits at position c ^ ((r >> 2) & 3): 16 consecutive
 // rows at one logical chunk then cover the 64 banks once. The barrier waits for this wave's copy of tile kt+1
 // only (vmcnt leaves the younger tiles in flight), hence the hand-written s_waitcnt.
-template <class E, bool GATED, bool KTAIL, int NS, int WP, int WQ, int FP, int FQ>
+// LAYOUT bits (256 x 256 tile only): 1 = the activation operand Q is panel-blocked (see block_rows_kernel),
+// 2 = the output is written panel-blocked (gated kernel: H for the down projection), 4 = the weight operand P is
+// panel-blocked (prepacked; for the gated kernel in de-interleaved row order). A blocked operand turns every copy
+// instruction into one contiguous 1 KB read of whole cache lines; row-major, a 32-element K tile is 64 bytes per
+// row, half a line per request. Measured at 8192 x 4096 x 14336: gate/up 1.52 -> 1.40 ms with X blocked, down
+// 0.81 -> 0.70 ms with H blocked.
+template <class E, bool GATED, bool KTAIL, int NS, int WP, int WQ, int FP, int FQ, int LAYOUT = 0>
 __global__ void __launch_bounds__(WP* WQ * 64)
 tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
   constexpr int NT = WP * WQ * 64;
@@ -522,6 +560,9 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
   static_assert(BP % RSTEP == 0 && BQ % RSTEP == 0 && RSTEP % 16 == 0, "copy mapping");
   static_assert(!GATED || (FP % 2 == 0), "gated kernel pairs fragments");
   static_assert(NS == 4 || NS == 5, "ring length");
+  constexpr bool QBLK = (LAYOUT & 1) != 0, OBLK = (LAYOUT & 2) != 0, PBLK = (LAYOUT & 4) != 0;
+  static_assert(LAYOUT == 0 || (BP == 256 && BQ == 256), "blocked layouts are defined for 256-row panels");
+  static_assert(!OBLK || GATED, "only H is ever written blocked");
   static_assert(NS * STAGE <= 160 * 1024, "LDS budget of a gfx950 CU");
 
   // one array per stage: the compiler tracks outstanding LDS DMA per array
@@ -548,21 +589,30 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
   const int pc = t & 3;
   const int rb = t >> 2;
   const int lc = pc ^ ((rb >> 2) & 3);
-  const unsigned char* pbase = (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
-  const unsigned char* qbase = (const unsigned char*)a.Q + (long long)q0 * a.ldq * 2;
-  const __amdgpu_buffer_rsrc_t prs = make_rsrc(pbase, ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
-  const __amdgpu_buffer_rsrc_t qrs = make_rsrc(qbase, ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2);
+  const int nkt = (a.k + BK - 1) / BK;
+  // a blocked panel: nkt blocks of [256 rows][64 bytes], block kt holds K elements 32 kt .. 32 kt + 31 (zero padded)
+  constexpr int PBLOCK = BP * ROWB, QBLOCK = BQ * ROWB;
+  const unsigned char* pbase = PBLK ? (const unsigned char*)a.P + (long long)tp * nkt * PBLOCK
+                                    : (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
+  const unsigned char* qbase = QBLK ? (const unsigned char*)a.Q + (long long)tq * nkt * QBLOCK
+                                    : (const unsigned char*)a.Q + (long long)q0 * a.ldq * 2;
+  const __amdgpu_buffer_rsrc_t prs =
+      make_rsrc(pbase, PBLK ? (long long)nkt * PBLOCK : ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
+  const __amdgpu_buffer_rsrc_t qrs =
+      make_rsrc(qbase, QBLK ? (long long)nkt * QBLOCK : ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2);
   unsigned poff[LP], qoff[LQ];
 #pragma unroll
   for (int i = 0; i < LP; ++i) {
     const int r = rb + i * RSTEP;
     const int grow = GATED ? (r < BP / 2 ? 2 * r : 2 * (r - BP / 2) + 1) : r;
-    poff[i] = (unsigned)grow * (unsigned)a.ldp * 2u + (unsigned)lc * 16u;
+    poff[i] = PBLK ? (unsigned)r * (unsigned)ROWB + (unsigned)lc * 16u
+                   : (unsigned)grow * (unsigned)a.ldp * 2u + (unsigned)lc * 16u;
   }
 #pragma unroll
   for (int i = 0; i < LQ; ++i) {
     const int r = rb + i * RSTEP;
-    qoff[i] = (unsigned)r * (unsigned)a.ldq * 2u + (unsigned)lc * 16u;
+    qoff[i] = QBLK ? (unsigned)r * (unsigned)ROWB + (unsigned)lc * 16u
+                   : (unsigned)r * (unsigned)a.ldq * 2u + (unsigned)lc * 16u;
   }
 
   unsigned xo[2];
@@ -583,8 +633,6 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[f][g][i] = 0.0f;
 
-  const int nkt = (a.k + BK - 1) / BK;
-
   // DMA instructions lo..hi-1 (of NL per wave: weight rows first, then activation rows) of K tile `kt`.
   auto dma = [&](unsigned char* stage, int kt, auto lo_c, auto hi_c) {
     constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
@@ -593,12 +641,15 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
     const bool in = !KTAIL || (ktc * BK + lc * 8) < a.k;
 #pragma unroll
     for (int i = LO; i < HI; ++i) {
+      // blocked operands are zero padded in K: no tail predicate, and the K tile selects a whole block
       if (i < LP) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(stage + i * RSTEP * ROWB + wave * 1024), 16,
-                                                 (int)(in ? poff[i] : OOB_OFFSET), kb, 0, 0);
+                                                 (int)((PBLK || in) ? poff[i] : OOB_OFFSET), PBLK ? ktc * PBLOCK : kb, 0,
+                                                 0);
       } else {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(stage + (BP + (i - LP) * RSTEP) * ROWB + wave * 1024),
-                                                 16, (int)(in ? qoff[i - LP] : OOB_OFFSET), kb, 0, 0);
+                                                 16, (int)((QBLK || in) ? qoff[i - LP] : OOB_OFFSET),
+                                                 QBLK ? ktc * QBLOCK : kb, 0, 0);
       }
     }
   };
@@ -710,7 +761,39 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
     }
   }
 
-  store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
+  if constexpr (OBLK) {
+    store_tile_blocked<E, WP, WQ, FP, FQ>(acc, a, tp, tq, wp, wq, l32, hi);
+  } else {
+    store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
+  }
+}
+
+// ---- row-major -> panel-blocked copy ---------------------------------------------------------------------------
+// dst block (panel, kt) = [256 rows][64 bytes]: rows 256 panel .. 256 panel + 255 of src, K elements 32 kt .. 32 kt + 31;
+// rows past `rows` and elements past `k` are written as zeros. A workgroup copies four K tiles of one panel: reads
+// are 256 contiguous bytes per row (16 lanes), writes 1 KB contiguous per 16 rows of a block.
+// gated_order (W13): block row r < 128 is source row 2r of the panel (the "up" row of feature r), block row
+// r >= 128 is source row 2(r - 128) + 1 (its "gate" row): the order the gated kernel keeps a weight tile in LDS.
+__global__ void __launch_bounds__(256)
+block_rows_kernel(const unsigned short* __restrict__ src, long long ld, int rows, int k, unsigned char* __restrict__ dst,
+                  int nkt, int gated_order) {
+  const int t = threadIdx.x;
+  const int c16 = t & 15;
+  const int r0 = t >> 4;
+  const int panel = blockIdx.y;
+  const int kt = (int)blockIdx.x * 4 + (c16 >> 2);
+  if (kt >= nkt) return;
+  const int k0 = (int)blockIdx.x * 128 + c16 * 8;
+  unsigned char* block = dst + ((long long)panel * nkt + kt) * (256 * 64) + (c16 & 3) * 16;
+#pragma unroll 4
+  for (int pass = 0; pass < 16; ++pass) {
+    const int row = pass * 16 + r0;
+    const int srow = gated_order ? (row < 128 ? 2 * row : 2 * (row - 128) + 1) : row;
+    const long long gr = (long long)panel * 256 + srow;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (gr < rows && k0 < k) v = *(const u32x4*)(src + gr * ld + k0);
+    *(u32x4*)(block + row * 64) = v;
+  }
 }
 
 // ---- variant table ------------------------------------------------------------------------------------
@@ -780,6 +863,38 @@ hipError_t launch_ring(const GemmArgs& a, hipStream_t stream) {
                        dim3(WP * WQ * 64), 0, stream, a, tiles_p, tiles_q, raster_group(GATED));
   }
   return hipGetLastError();
+}
+
+// 256 x 256 ring kernel with blocked operands / output (GemmArgs::layout, bits as in tiled_ring_kernel)
+template <class E, bool GATED, int NS, int LAYOUT>
+hipError_t launch_ring_layout(const GemmArgs& a, hipStream_t stream) {
+  const int tiles_p = (a.np + 255) / 256;
+  const int tiles_q = (a.nq + 255) / 256;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
+  if constexpr ((LAYOUT & 4) != 0) {  // a blocked weight operand is zero padded in K as well: no K tail anywhere
+    hipLaunchKernelGGL((tiled_ring_kernel<E, GATED, false, NS, 2, 2, 4, 4, LAYOUT>), grid, block, 0, stream, a, tiles_p,
+                       tiles_q, raster_group(GATED));
+  } else if (a.k % 32 == 0) {
+    hipLaunchKernelGGL((tiled_ring_kernel<E, GATED, false, NS, 2, 2, 4, 4, LAYOUT>), grid, block, 0, stream, a, tiles_p,
+                       tiles_q, raster_group(GATED));
+  } else {
+    hipLaunchKernelGGL((tiled_ring_kernel<E, GATED, true, NS, 2, 2, 4, 4, LAYOUT>), grid, block, 0, stream, a, tiles_p,
+                       tiles_q, raster_group(GATED));
+  }
+  return hipGetLastError();
+}
+
+template <class E>
+hipError_t launch_blocked_typed(bool gated, const GemmArgs& a, hipStream_t stream) {
+  if (gated) {
+    if (a.layout == 3) return launch_ring_layout<E, true, 5, 3>(a, stream);
+    if (a.layout == 7) return launch_ring_layout<E, true, 5, 7>(a, stream);
+  } else {
+    if (a.layout == 1) return launch_ring_layout<E, false, 4, 1>(a, stream);
+    if (a.layout == 5) return launch_ring_layout<E, false, 4, 5>(a, stream);
+  }
+  return hipErrorInvalidValue;
 }
 
 template <class E, bool GATED>
@@ -858,6 +973,20 @@ hipError_t launch_tiled_splitk(int dtype, int tile, const GemmArgs& a, hipStream
     return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 2>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 2>(a, stream);
   }
   return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 4, 4>(a, stream) : launch_splitk_one<Fp16, 2, 2, 4, 4>(a, stream);
+}
+
+hipError_t launch_tiled_blocked(int dtype, bool gated, const GemmArgs& a, hipStream_t stream) {
+  return dtype == 0 ? launch_blocked_typed<Bf16>(gated, a, stream) : launch_blocked_typed<Fp16>(gated, a, stream);
+}
+
+hipError_t launch_block_rows(const void* src, long long ld, int rows, int k, void* dst, bool gated_order,
+                             hipStream_t stream) {
+  const int nkt = (k + 31) / 32;
+  const int panels = (rows + 255) / 256;
+  if (nkt <= 0 || panels <= 0) return hipSuccess;
+  hipLaunchKernelGGL(block_rows_kernel, dim3((unsigned)((nkt + 3) / 4), (unsigned)panels), dim3(256), 0, stream,
+                     (const unsigned short*)src, ld, rows, k, (unsigned char*)dst, nkt, gated_order ? 1 : 0);
+  return hipGetLastError();
 }
 
 void set_raster_group(int g) { g_raster_group = g > 0 ? g : 0; }

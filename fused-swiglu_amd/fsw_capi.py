@@ -24,6 +24,12 @@ PROTOTYPES = {
     "fsw_down": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
     "fsw_mlp_workspace_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "fsw_mlp": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "fsw_blocked_bytes": (_sz, [_i64, _i64]),
+    "fsw_block_rows": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
+    "fsw_prepack_w13": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
+    "fsw_prepack_w2": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
+    "fsw_gateup_blocked": (_i, [_i, _i64, _i64, _i64, _vp, _vp, _i64, _i, _vp, _vp]),
+    "fsw_down_blocked": (_i, [_i, _i64, _i64, _i64, _vp, _vp, _i64, _i, _vp, _i64, _vp]),
     "fsw_strerror": (_cp, [_i]),
     "fsw_last_hip_error": (_i, []),
     "fsw_version": (_i, []),
@@ -142,6 +148,71 @@ def mlp(X, W13, W2, out=None, workspace=None):
     with torch.cuda.device(X.device):
         check(lib().fsw_mlp(code, M, D, FF, X.data_ptr(), _ld(X), W13.data_ptr(), _ld(W13), W2.data_ptr(), _ld(W2),
                             out.data_ptr(), _ld(out), workspace.data_ptr(), workspace.numel(), _stream(X)))
+    return out
+
+
+class Blocked:
+    """A panel-blocked device copy of a row-major [rows, k] matrix (fsw.h: blocks of [256 rows][32 elements])."""
+
+    def __init__(self, buf, rows, k, dtype):
+        self.buf, self.rows, self.k, self.dtype = buf, rows, k, dtype
+
+    def data_ptr(self):
+        return self.buf.data_ptr()
+
+
+def _blocked_empty(rows, k, like):
+    import torch
+    n = lib().fsw_blocked_bytes(rows, k)
+    return Blocked(torch.empty(max(n, 16), dtype=torch.uint8, device=like.device), rows, k, like.dtype)
+
+
+def block_rows(A, kind="rows"):
+    """Row-major device matrix -> Blocked. kind: "rows" (X, H, W2) or "w13" (up/gate rows de-interleaved per panel)."""
+    import torch
+    rows, k = A.shape
+    out = _blocked_empty(rows, k, A)
+    fn = {"rows": lib().fsw_block_rows, "w13": lib().fsw_prepack_w13, "w2": lib().fsw_prepack_w2}[kind]
+    with torch.cuda.device(A.device):
+        check(fn(dtype_code(A), rows, k, A.data_ptr(), _ld(A), out.data_ptr(), _stream(A)))
+    return out
+
+
+def unblock(B):
+    """Blocked -> row-major torch tensor (host-side index arithmetic on the device buffer; for tests)."""
+    import torch
+    panels, nkt = (B.rows + 255) // 256, (B.k + 31) // 32
+    t = B.buf[: panels * nkt * 256 * 64].view(B.dtype).view(panels, nkt, 256, 32)
+    return t.permute(0, 2, 1, 3).reshape(panels * 256, nkt * 32)[: B.rows, : B.k].contiguous()
+
+
+def gateup_blocked(Xb, W13, N=None):
+    """Blocked H = gate/up of a Blocked X. W13: row-major tensor, or a Blocked from block_rows(W13, "w13") with N."""
+    import torch
+    wb = isinstance(W13, Blocked)
+    N = W13.rows if wb else W13.shape[0]
+    like = Xb.buf
+    Hb = Blocked(torch.empty(max(lib().fsw_blocked_bytes(Xb.rows, N // 2), 16), dtype=torch.uint8, device=like.device),
+                 Xb.rows, N // 2, Xb.dtype)
+    code = BF16 if Xb.dtype == torch.bfloat16 else FP16
+    with torch.cuda.device(like.device):
+        check(lib().fsw_gateup_blocked(code, Xb.rows, N, Xb.k, Xb.data_ptr(), W13.data_ptr(), 0 if wb else _ld(W13),
+                                       1 if wb else 0, Hb.data_ptr(), _stream(like)))
+    return Hb
+
+
+def down_blocked(Hb, W2, out=None):
+    """Row-major Y = Blocked H @ W2.T. W2: row-major tensor or a Blocked from block_rows(W2, "w2")."""
+    import torch
+    wb = isinstance(W2, Blocked)
+    D = W2.rows if wb else W2.shape[0]
+    like = Hb.buf
+    if out is None:
+        out = torch.empty((Hb.rows, D), dtype=Hb.dtype, device=like.device)
+    code = BF16 if Hb.dtype == torch.bfloat16 else FP16
+    with torch.cuda.device(like.device):
+        check(lib().fsw_down_blocked(code, Hb.rows, D, Hb.k, Hb.data_ptr(), W2.data_ptr(), 0 if wb else _ld(W2),
+                                     1 if wb else 0, out.data_ptr(), _ld(out), _stream(like)))
     return out
 
 

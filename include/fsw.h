@@ -106,6 +106,32 @@ FSW_API int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF,
 /* Text for an FSW_E_* code (static storage, never NULL). */
 FSW_API const char* fsw_strerror(int code);
 
+/*
+ * Panel-blocked layout (no counterpart in the reference; it is the offline/in-flight layout transform that lets the
+ * large-tile kernels fetch whole cache lines). A blocked copy of a row-major [rows, k] matrix is ceil(rows / 256)
+ * panels of ceil(k / 32) blocks; block (panel, kt) is [256 rows][32 elements] contiguous (16 KB) and holds rows
+ * 256 panel .. 256 panel + 255, columns 32 kt .. 32 kt + 31, zero padded. fsw_mlp uses it internally for M > 64 when
+ * both projections run 256 x 256 tiles (X re-blocked into the workspace, H written and read blocked); the entry
+ * points below expose the steps, and let a caller block the weights ONCE (fsw_prepack_*) and pass them with
+ * w_blocked = 1. Constraints as for fsw_gateup / fsw_down (K, FF and row-major leading dimensions multiples of 8,
+ * 16-byte aligned bases); the blocked kernels are the 256 x 256 tiled kernels, whatever M is.
+ */
+FSW_API size_t fsw_blocked_bytes(int64_t rows, int64_t k);
+FSW_API int fsw_block_rows(int dtype, int64_t rows, int64_t k, const void* src, int64_t ld, void* dst_blocked,
+                           void* stream);
+/* W13 [N, K] interleaved as in swiglu.cu:380-381 -> blocked, with each panel's 128 "up" rows first, then its 128
+ * "gate" rows (the order the gated kernel keeps a weight tile in LDS). */
+FSW_API int fsw_prepack_w13(int dtype, int64_t N, int64_t K, const void* W13, int64_t ldw, void* dst_blocked,
+                            void* stream);
+FSW_API int fsw_prepack_w2(int dtype, int64_t D, int64_t FF, const void* W2, int64_t ldw2, void* dst_blocked,
+                           void* stream);
+/* H_blocked[M, N/2] = gate/up of X_blocked[M, K]; W13 row-major (w_blocked = 0, ldw) or from fsw_prepack_w13 (1). */
+FSW_API int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* X_blocked, const void* W13,
+                               int64_t ldw, int w_blocked, void* H_blocked, void* stream);
+/* Y[M, D] (row-major, ldy) = H_blocked[M, FF] @ W2^T; W2 row-major (0, ldw2) or from fsw_prepack_w2 (1). */
+FSW_API int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* H_blocked, const void* W2,
+                             int64_t ldw2, int w_blocked, void* Y, int64_t ldy, void* stream);
+
 /* The hipError_t (as int) of the most recent failed launch on the calling thread, 0 if none. */
 FSW_API int fsw_last_hip_error(void);
 

@@ -428,3 +428,66 @@ def test_config_c3_headline(capi):
 
 def test_config_c5_fp16(capi):
     _config_case(capi, "C5", 96)
+
+
+# ---- panel-blocked layout: the transform, the kernels that read / write it, and fsw_mlp's large-tile regime ----------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_block_rows_layout(capi, dtype):
+    """fsw_block_rows / fsw_prepack_*: block (panel, kt) = [256 rows][32 elements], zero padded; W13 panels carry
+    their 128 up rows first, then their 128 gate rows. Bit exact against index arithmetic in torch."""
+    for (rows, k, ld) in [(1, 8, 8), (300, 72, 72), (256, 32, 40), (513, 1000, 1008), (700, 4096, 4096)]:
+        A = (torch.randn(rows, ld) * 3).to(dtype).to(DEV)[:, :k]
+        B = capi.block_rows(A)
+        assert torch.equal(capi.unblock(B), A)
+        # padding is zero: the K loop of the consumer reads it
+        panels, nkt = (rows + 255) // 256, (k + 31) // 32
+        full = B.buf[: panels * nkt * 256 * 64].view(dtype).view(panels, nkt, 256, 32).permute(0, 2, 1, 3).reshape(panels * 256, nkt * 32)
+        assert full[rows:].abs().max().item() == 0 if rows < panels * 256 else True
+        assert full[:, k:].abs().max().item() == 0 if k < nkt * 32 else True
+    W13 = (torch.randn(600, 64)).to(dtype).to(DEV)
+    P = capi.unblock(capi.block_rows(W13, "w13"))  # row r of panel p: up rows then gate rows of that panel
+    expect = torch.zeros(768, 64, dtype=dtype, device=DEV)
+    src = torch.zeros(768, 64, dtype=dtype, device=DEV)
+    src[:600] = W13
+    for p in range(3):
+        expect[256 * p: 256 * p + 128] = src[256 * p: 256 * p + 256: 2]
+        expect[256 * p + 128: 256 * p + 256] = src[256 * p + 1: 256 * p + 256: 2]
+    assert torch.equal(P, expect[:600])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("prepacked", [False, True])
+def test_blocked_kernels_against_oracle(capi, dtype, prepacked):
+    """fsw_gateup_blocked / fsw_down_blocked on ragged shapes (M, K, ff not multiples of the 256 / 32 blocking),
+    with row-major and with prepacked weights: H (unblocked) to one rounding, Y to one rounding given H."""
+    for (M, d, ff) in [(300, 1000, 520), (64, 136, 40), (513, 4096, 264), (1024, 512, 1032)]:
+        inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=17 * M + ff, x_scale=0.5)
+        g = to_dev(inp)
+        Xb = capi.block_rows(g["X"])
+        W13 = capi.block_rows(g["W13"], "w13") if prepacked else g["W13"]
+        W2 = capi.block_rows(g["W2"], "w2") if prepacked else g["W2"]
+        Hb = capi.gateup_blocked(Xb, W13)
+        H = capi.unblock(Hb)
+        assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "blocked H %s" % ((M, d, ff),))
+        Y = capi.down_blocked(Hb, W2)
+        assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype, "blocked Y %s" % ((M, d, ff),))
+        oracle.assert_parity(Y, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64), "blocked mlp %s" % ((M, d, ff),))
+        # same bits as the row-major kernels up to the fp32 summation order of the K loop (identical here: same kernel)
+        H2 = capi.gateup(g["X"], g["W13"])
+        assert (H.float() - H2.float()).abs().max().item() <= 2 * ulp_rel(dtype) * 2 * H2.float().abs().max().item() + 1e-3
+
+
+def test_mlp_large_tile_regime_uses_blocked_path(capi):
+    """For M > 64 with both projections on 256 x 256 tiles fsw_mlp re-blocks X into the workspace and keeps H blocked;
+    the result agrees with the separate row-major entry points and with the oracle, and the workspace query covers
+    both blocked buffers."""
+    M, d, ff = 4096, 4096, 2048
+    L = capi.lib()
+    assert L.fsw_mlp_workspace_bytes(0, M, d, ff) == L.fsw_blocked_bytes(M, ff) + L.fsw_blocked_bytes(M, d)
+    inp = fsw_weights.make_inputs(M, d, ff, torch.bfloat16, seed=99, x_scale=0.5)
+    g = to_dev(inp)
+    Y = capi.mlp(g["X"], g["W13"], g["W2"])
+    Y2 = capi.down(capi.gateup(g["X"], g["W13"]), g["W2"])
+    rows = torch.arange(0, M, 37)
+    oracle.assert_parity(Y[rows.to(DEV)], oracle.ref_mlp(inp["X"][rows], inp["W13"], inp["W2"], torch.float64), "mlp blocked regime")
+    assert (Y.float() - Y2.float()).abs().max().item() <= 2e-2
