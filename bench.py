@@ -47,17 +47,21 @@ def parse():
                     help="also run one elementwise copy of 1 GiB (reads 1 GiB, writes 1 GiB): the known-size kernel "
                          "that FETCH_SIZE / WRITE_SIZE counter runs are scaled by")
     ap.add_argument("--no-decode", action="store_true", help="skip the M=16 decode leg")
+    ap.add_argument("--no-prepacked", action="store_true", help="skip the leg with weights blocked offline")
     return ap.parse_args()
 
 
-def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False):
+def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False, prepacked=False):
     """Times exactly `steps` forwards between two device synchronisations.
-    fused_entry=False: a step is fsw_gateup followed by fsw_down (exactly what fsw_mlp enqueues for M > 64), with
-    HIP events recorded around each launch inside the timed region.
+    fused_entry=False: a step is the launch sequence fsw_mlp enqueues for this shape, issued through the
+    per-step entry points so that HIP events can be recorded around each launch inside the timed region: in the
+    large-tile regime fsw_block_rows(X) -> fsw_gateup_blocked -> fsw_down_blocked (H stays blocked in the
+    workspace), otherwise fsw_gateup -> fsw_down. prepacked=True passes weights blocked once, outside the timed
+    region, by fsw_prepack_w13 / fsw_prepack_w2.
     fused_entry=True: a step is one fsw_mlp call and ONE event pair brackets the whole timed region (an event
     record costs the stream ~4 us, which is 6 % of a 64 us decode step but 0.2 % of a prefill step); the per-step
     kernel time is then the bracketed time / steps, inter-launch gaps included.
-    Returns (wall seconds, [ms of first interval], [ms of second interval], Y)."""
+    Returns (wall seconds, [ms of gate/up], [ms of down], Y, [ms of the X re-block or 0])."""
     import fsw_capi
     L = capi.lib()
     M, d, ff = cfg["M"], cfg["d"], cfg["ff"]
@@ -66,23 +70,40 @@ def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False):
     ws_bytes = L.fsw_mlp_workspace_bytes(code, M, d, ff)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=g["X"].device)
     h_bytes = (M * ff * 2 + 255) // 256 * 256
+    hb_bytes = L.fsw_blocked_bytes(M, ff)
+    blocked = (not fused_entry) and ws_bytes == hb_bytes + L.fsw_blocked_bytes(M, d)
     stream = torch.cuda.current_stream().cuda_stream
     xp, wp, w2p, yp, wsp = (t.data_ptr() for t in (g["X"], g["W13"], g["W2"], Y, ws))
+    ldw, ldw2, wflag = d, ff, 0
+    if prepacked:
+        if not blocked:
+            raise RuntimeError("prepacked weights are only used in the large-tile regime")
+        w13b, w2b = capi.block_rows(g["W13"], "w13"), capi.block_rows(g["W2"], "w2")
+        wp, w2p, ldw, ldw2, wflag = w13b.data_ptr(), w2b.data_ptr(), 0, 0, 1
 
     def step(ev):
         if fused_entry:
             rc = L.fsw_mlp(code, M, d, ff, xp, d, wp, d, w2p, ff, yp, d, wsp, ws_bytes, stream)
-            rc2 = 0
+            rc2 = rc3 = 0
+        elif blocked:
+            ev[3].record()
+            rc3 = L.fsw_block_rows(code, M, d, xp, d, wsp + hb_bytes, stream)
+            ev[0].record()
+            rc = L.fsw_gateup_blocked(code, M, 2 * ff, d, wsp + hb_bytes, wp, ldw, wflag, wsp, 0, stream)
+            ev[1].record()
+            rc2 = L.fsw_down_blocked(code, M, d, ff, wsp, w2p, ldw2, wflag, yp, d, stream)
+            ev[2].record()
         else:
             ev[0].record()
             rc = L.fsw_gateup(code, M, 2 * ff, d, xp, d, wp, d, wsp, ff, stream)
             ev[1].record()
             rc2 = L.fsw_down(code, M, d, ff, wsp, ff, w2p, ff, yp, d, wsp + h_bytes, ws_bytes - h_bytes, stream)
             ev[2].record()
-        if rc or rc2:
-            raise RuntimeError("fsw launch failed: %s / %s" % (capi.strerror(rc), capi.strerror(rc2)))
+            rc3 = 0
+        if rc or rc2 or rc3:
+            raise RuntimeError("fsw launch failed: %s / %s / %s" % (capi.strerror(rc), capi.strerror(rc2), capi.strerror(rc3)))
 
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps + warmup)]
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps + warmup)]
     region = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
     for i in range(warmup):
         step(events[steps + i])
@@ -95,10 +116,11 @@ def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     if fused_entry:
-        return wall, [region[0].elapsed_time(region[1]) / steps], [0.0], Y
+        return wall, [region[0].elapsed_time(region[1]) / steps], [0.0], Y, [0.0]
     first = [e[0].elapsed_time(e[1]) for e in events[:steps]]
     second = [e[1].elapsed_time(e[2]) for e in events[:steps]]
-    return wall, first, second, Y
+    pre = [e[3].elapsed_time(e[0]) for e in events[:steps]] if blocked else [0.0]
+    return wall, first, second, Y, pre
 
 
 def cpu_baseline(torch, inp, cfg, budget_s, y_gpu):
@@ -159,7 +181,9 @@ def main():
     M, d, ff = cfg["M"], cfg["d"], cfg["ff"]
     dtype_name = "bf16" if inp["dtype"] == torch.bfloat16 else "fp16"
     hbm_bound = args.workload == "C4"
-    wall, gu, dn, Y = run_steps(capi, torch, g, cfg, args.steps, args.warmup, fused_entry=hbm_bound)
+    wall, gu, dn, Y, pre = run_steps(capi, torch, g, cfg, args.steps, args.warmup, fused_entry=hbm_bound)
+    pre_ms = sum(pre) / len(pre)
+    blocked = pre_ms > 0
     ms_per_step = wall / args.steps * 1e3
     tflops = fsw_weights.flops(M, d, ff) / (ms_per_step * 1e-3) / 1e12
     gu_ms, dn_ms = sum(gu) / len(gu), max(sum(dn) / len(dn), 1e-9)
@@ -173,7 +197,8 @@ def main():
                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "algorithmic_bytes": all_bytes,
                     "avg_kernel_ms": round(gu_ms, 5)}
     else:
-        roofline = {"bound": "mfma", "kernel": capi.variant_name(0, 0, M, 2 * ff, d) + " (gate/up)",
+        kname = "ring5_256x256, X and H panel-blocked" if blocked else capi.variant_name(0, 0, M, 2 * ff, d)
+        roofline = {"bound": "mfma", "kernel": kname + " (gate/up)",
                     "achieved": round(gu_tflops, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(gu_tflops / MFMA_PEAK_TFLOPS, 4),
                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
@@ -188,7 +213,7 @@ def main():
         "frac_of_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS, 4),
         "kernels": {"gateup_ms": round(gu_ms, 5), "gateup_ms_median": round(med(gu), 5),
                     "gateup_tflops": round(gu_tflops, 2), "down_ms": round(dn_ms, 5),
-                    "down_tflops": round(dn_tflops, 2),
+                    "down_tflops": round(dn_tflops, 2), "block_x_ms": round(pre_ms, 5),
                     "hbm_gbs": round(fsw_weights.hbm_bytes(M, d, ff) / (ms_per_step * 1e-3) / 1e9, 2)},
         "roofline": roofline,
     }
@@ -204,7 +229,7 @@ def main():
     if args.workload != "C4" and not args.no_decode:
         inp4, g4 = load("C4")
         c4 = {k: inp4[k] for k in ("name", "M", "d", "ff", "seed")}
-        wall4, k4, _, _ = run_steps(capi, torch, g4, c4, 200, 20, fused_entry=True)  # one fsw_mlp call per step
+        wall4, k4, _, _, _ = run_steps(capi, torch, g4, c4, 200, 20, fused_entry=True)  # one fsw_mlp call per step
         ms4 = wall4 / 200 * 1e3
         k4_ms = sum(k4) / len(k4)
         by4 = fsw_weights.hbm_bytes(c4["M"], c4["d"], c4["ff"])
@@ -217,12 +242,23 @@ def main():
                                       "traffic": None, "avg_kernel_ms": round(k4_ms, 5)}}
         del inp4, g4
 
+    # the same forward with the weights blocked once, offline (fsw_prepack_w13 / fsw_prepack_w2): reported beside
+    # `value`, which stays on the reference's weight layout
+    if blocked and not args.no_prepacked:
+        wallp, gup, dnp, Yp, prep = run_steps(capi, torch, g, cfg, args.steps, args.warmup, prepacked=True)
+        msp = wallp / args.steps * 1e3
+        out["prepacked_weights"] = {
+            "ms_per_step": round(msp, 5), "value": round(fsw_weights.flops(M, d, ff) / (msp * 1e-3) / 1e12, 2),
+            "unit": "TFLOP/s", "gateup_ms": round(sum(gup) / len(gup), 5), "down_ms": round(sum(dnp) / len(dnp), 5),
+            "block_x_ms": round(sum(prep) / len(prep), 5),
+            "max_abs_vs_row_major_weights": round((Yp.float() - Y.float()).abs().max().item(), 6)}
+
     if args.detail:
         for name in ("C1", "C2", "C3", "C4", "C5"):
             i2, g2 = load(name)
             c2 = {k: i2[k] for k in ("name", "M", "d", "ff", "seed")}
             n = 200 if name in ("C1", "C4") else 30
-            w2, a2, b2, _ = run_steps(capi, torch, g2, c2, n, 5, fused_entry=(name == "C4"))
+            w2, a2, b2, _, _ = run_steps(capi, torch, g2, c2, n, 5, fused_entry=(name == "C4"))
             ms2 = w2 / n * 1e3
             print("%s  %.4f ms/step  %.1f TFLOP/s  %.1f GB/s  gate/up %.4f ms  down %.4f ms" % (
                 name, ms2, fsw_weights.flops(c2["M"], c2["d"], c2["ff"]) / ms2 / 1e9,

@@ -287,7 +287,7 @@ int fsw_prepack_w2(int dtype, int64_t D, int64_t FF, const void* W2, int64_t ldw
 }
 
 int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* Xb, const void* W13, int64_t ldw,
-                       int w_blocked, void* Hb, void* stream) {
+                       int w_blocked, void* Hb, int64_t ldh, void* stream) {
   if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
   if (M < 0 || N < 0 || K < 0 || (N & 1) || M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return FSW_E_SHAPE;
   if (M == 0 || N == 0) return FSW_OK;
@@ -295,8 +295,10 @@ int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* X
   if (!Xb || !W13 || !Hb) return FSW_E_NULL;
   if (!w_blocked && ldw < K) return FSW_E_LD;
   if (!w_blocked && ldw > MAX_LD) return FSW_E_SHAPE;
+  if (ldh != 0 && ldh < N / 2) return FSW_E_LD;
+  if (ldh > MAX_DIM) return FSW_E_SHAPE;
   if ((K & 7) || (!w_blocked && (ldw & 7))) return FSW_E_ALIGN;
-  if (!aligned16(Xb) || !aligned16(W13) || !aligned16(Hb)) return FSW_E_ALIGN;
+  if (!aligned16(Xb) || !aligned16(W13) || (ldh == 0 ? !aligned16(Hb) : ((((uintptr_t)Hb) & 1) != 0))) return FSW_E_ALIGN;
   const int drc = check_device();
   if (drc != FSW_OK) return drc;
   fsw::GemmArgs a;
@@ -305,11 +307,11 @@ int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* X
   a.O = Hb;
   a.ldp = ldw;
   a.ldq = 0;
-  a.ldo = 0;
+  a.ldo = ldh;
   a.np = (int)N;
   a.nq = (int)M;
   a.k = (int)K;
-  a.layout = w_blocked ? 7 : 3;
+  a.layout = 1 | (ldh == 0 ? 2 : 0) | (w_blocked ? 4 : 0);
   return finish(fsw::launch_tiled_blocked(dtype, true, a, (hipStream_t)stream));
 }
 
@@ -338,6 +340,28 @@ int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* Hb
   a.k = (int)FF;
   a.layout = w_blocked ? 5 : 1;
   return finish(fsw::launch_tiled_blocked(dtype, false, a, (hipStream_t)stream));
+}
+
+// fsw_gateup with caller scratch: in the large-tile regime X is re-blocked into the scratch first (the gated
+// kernel then reads whole cache lines: 1.52 -> 1.40 + 0.03 ms at 8192 x 4096 x 28672); H stays row-major.
+size_t fsw_gateup_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K) {
+  (void)dtype;
+  if (M <= 64 || N <= 0 || K <= 0 || M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return 0;
+  if (g_forced_variant[0] >= 0 || pick_tiled(0, M, N) != 8) return 0;
+  return (size_t)fsw::blocked_bytes(M, K);
+}
+
+int fsw_gateup_ws(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13, int64_t ldw,
+                  void* H, int64_t ldh, void* workspace, size_t workspace_bytes, void* stream) {
+  const size_t want = fsw_gateup_workspace_bytes(dtype, M, N, K);
+  if (want == 0 || !workspace || workspace_bytes < want || !aligned16(workspace)) {
+    return fsw_gateup(dtype, M, N, K, X, ldx, W13, ldw, H, ldh, stream);
+  }
+  int rc = fsw_validate_gateup(dtype, M, N, K, X, ldx, W13, ldw, H, ldh);
+  if (rc != FSW_OK) return rc;
+  rc = fsw_block_rows(dtype, M, K, X, ldx, workspace, stream);
+  if (rc != FSW_OK) return rc;
+  return fsw_gateup_blocked(dtype, M, N, K, workspace, W13, ldw, 0, H, ldh, stream);
 }
 
 static size_t h_bytes(int64_t M, int64_t FF) {
@@ -394,7 +418,7 @@ int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t 
     unsigned char* Xb = Hb + fsw::blocked_bytes(M, FF);
     rc = fsw_block_rows(dtype, M, D, X, ldx, Xb, stream);
     if (rc != FSW_OK) return rc;
-    rc = fsw_gateup_blocked(dtype, M, 2 * FF, D, Xb, W13, ldw13, 0, Hb, stream);
+    rc = fsw_gateup_blocked(dtype, M, 2 * FF, D, Xb, W13, ldw13, 0, Hb, 0, stream);
     if (rc != FSW_OK) return rc;
     return fsw_down_blocked(dtype, M, D, FF, Hb, W2, ldw2, 0, Y, ldy, stream);
   }

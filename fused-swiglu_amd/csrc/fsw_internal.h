@@ -39,7 +39,8 @@ void set_raster_group(int g);  // activation-row tiles per raster band; 0 restor
 int tiled_variant_count();
 const TiledVariant& tiled_variant(int variant);
 hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
-// gated: layout 3 (X blocked in, H blocked out) or 7 (+ W13 blocked); plain: layout 1 (H blocked in) or 5 (+ W2 blocked)
+// gated: X blocked in (bit 0), H blocked out (bit 1) or row-major, W13 blocked (bit 2) or row-major: layouts 1, 3, 5, 7;
+// plain: H blocked in, W2 row-major (1) or blocked (5)
 hipError_t launch_tiled_blocked(int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
 // row-major [rows, k] (row stride ld elements) -> blocked; gated_order: W13's up/gate rows de-interleaved per panel
 hipError_t launch_block_rows(const void* src, long long ld, int rows, int k, void* dst, bool gated_order,

@@ -888,7 +888,9 @@ hipError_t launch_ring_layout(const GemmArgs& a, hipStream_t stream) {
 template <class E>
 hipError_t launch_blocked_typed(bool gated, const GemmArgs& a, hipStream_t stream) {
   if (gated) {
+    if (a.layout == 1) return launch_ring_layout<E, true, 5, 1>(a, stream);
     if (a.layout == 3) return launch_ring_layout<E, true, 5, 3>(a, stream);
+    if (a.layout == 5) return launch_ring_layout<E, true, 5, 5>(a, stream);
     if (a.layout == 7) return launch_ring_layout<E, true, 5, 7>(a, stream);
   } else {
     if (a.layout == 1) return launch_ring_layout<E, false, 4, 1>(a, stream);

@@ -13,6 +13,8 @@
 #include <torch/all.h>
 #include <torch/extension.h>
 
+#include <algorithm>
+
 #include "fsw.h"
 
 namespace {
@@ -51,8 +53,12 @@ void swiglu_fwd_typed(at::ScalarType want, int64_t m, int64_t n, int64_t k, Tens
     TORCH_CHECK(C.numel() >= (m - 1) * (ldC / 2) + n / 2, "tensor C is smaller than m x n/2 with row stride ldC/2");
   }
   const at::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(A));
-  const int rc = fsw_gateup(dtype_code(want), m, n, k, A.data_ptr(), ldA, B.data_ptr(), ldB, C.data_ptr(), ldC / 2,
-                            current_stream());
+  // large problems: scratch for a blocked copy of A lets the kernel fetch whole cache lines (same result)
+  const size_t ws_bytes = fsw_gateup_workspace_bytes(dtype_code(want), m, n, k);
+  Tensor ws;
+  if (ws_bytes > 0) ws = at::empty({(int64_t)ws_bytes}, A.options().dtype(at::kByte));
+  const int rc = fsw_gateup_ws(dtype_code(want), m, n, k, A.data_ptr(), ldA, B.data_ptr(), ldB, C.data_ptr(), ldC / 2,
+                               ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, current_stream());
   check_rc(rc, "swiglu_fwd");
 }
 
@@ -111,8 +117,29 @@ Tensor swiglu_down_fp16(Tensor const& H, Tensor const& W2) { return swiglu_down_
 
 // Y = (silu(X @ Wg) * (X @ Wu)) @ Wd with W1W3 = interleaved [up; gate] rows and W2 = Wd^T.
 Tensor fused_swiglu_mlp_typed(at::ScalarType want, Tensor const& X, Tensor const& W1W3, Tensor const& W2) {
-  Tensor H = fused_swiglu_typed(want, X, W1W3);
-  return swiglu_down_typed(want, H, W2);
+  TORCH_CHECK(X.scalar_type() == want && W1W3.scalar_type() == want && W2.scalar_type() == want,
+              "Expected tensors X, W1W3 and W2 to be of type ", want);
+  check_device_tensor(X, "X");
+  check_device_tensor(W1W3, "W1W3");
+  check_device_tensor(W2, "W2");
+  TORCH_CHECK(X.device() == W1W3.device() && X.device() == W2.device(), "X, W1W3 and W2 must live on the same device");
+  TORCH_CHECK(X.dim() == 2 && W1W3.dim() == 2 && W2.dim() == 2, "X, W1W3 and W2 must be 2-D");
+  const int64_t M = X.size(0), D = X.size(1), N = W1W3.size(0), FF = N / 2;
+  TORCH_CHECK(N % 2 == 0 && W1W3.size(1) == D, "W1W3 must be [2*ff, d] for X [M, d]");
+  TORCH_CHECK(W2.size(0) == D && W2.size(1) == FF, "W2 must be [d, ff]");
+  TORCH_CHECK((X.stride(1) == 1 || D <= 1) && (W1W3.stride(1) == 1 || D <= 1) && (W2.stride(1) == 1 || FF <= 1),
+              "X, W1W3 and W2 must be contiguous in their last dimension");
+  Tensor Y = at::empty({M, D}, X.options());
+  const at::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(X));
+  const int code = dtype_code(want);
+  // one call: H (and, for large problems, a blocked copy of X) live in this scratch, never as a tensor
+  const size_t ws_bytes = fsw_mlp_workspace_bytes(code, M, D, FF);
+  Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 16)}, X.options().dtype(at::kByte));
+  const int rc = fsw_mlp(code, M, D, FF, X.data_ptr(), M > 1 ? X.stride(0) : D, W1W3.data_ptr(),
+                         N > 1 ? W1W3.stride(0) : D, W2.data_ptr(), D > 1 ? W2.stride(0) : FF, Y.data_ptr(), D,
+                         ws.data_ptr(), ws_bytes, current_stream());
+  check_rc(rc, "fused_swiglu_mlp");
+  return Y;
 }
 
 Tensor fused_swiglu_mlp_bf16(Tensor const& X, Tensor const& W1W3, Tensor const& W2) {

@@ -28,8 +28,10 @@ PROTOTYPES = {
     "fsw_block_rows": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
     "fsw_prepack_w13": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
     "fsw_prepack_w2": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
-    "fsw_gateup_blocked": (_i, [_i, _i64, _i64, _i64, _vp, _vp, _i64, _i, _vp, _vp]),
+    "fsw_gateup_blocked": (_i, [_i, _i64, _i64, _i64, _vp, _vp, _i64, _i, _vp, _i64, _vp]),
     "fsw_down_blocked": (_i, [_i, _i64, _i64, _i64, _vp, _vp, _i64, _i, _vp, _i64, _vp]),
+    "fsw_gateup_workspace_bytes": (_sz, [_i, _i64, _i64, _i64]),
+    "fsw_gateup_ws": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
     "fsw_strerror": (_cp, [_i]),
     "fsw_last_hip_error": (_i, []),
     "fsw_version": (_i, []),
@@ -102,9 +104,11 @@ def gateup(X, W13, out=None):
     N = W13.shape[0]
     if out is None:
         out = torch.empty((M, N // 2), dtype=X.dtype, device=X.device)
+    nbytes = lib().fsw_gateup_workspace_bytes(code, M, N, K)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device) if nbytes else None
     with torch.cuda.device(X.device):
-        check(lib().fsw_gateup(code, M, N, K, X.data_ptr(), _ld(X), W13.data_ptr(), _ld(W13), out.data_ptr(),
-                               _ld(out), _stream(X)))
+        check(lib().fsw_gateup_ws(code, M, N, K, X.data_ptr(), _ld(X), W13.data_ptr(), _ld(W13), out.data_ptr(),
+                                  _ld(out), ws.data_ptr() if ws is not None else None, nbytes, _stream(X)))
     return out
 
 
@@ -186,19 +190,25 @@ def unblock(B):
     return t.permute(0, 2, 1, 3).reshape(panels * 256, nkt * 32)[: B.rows, : B.k].contiguous()
 
 
-def gateup_blocked(Xb, W13, N=None):
-    """Blocked H = gate/up of a Blocked X. W13: row-major tensor, or a Blocked from block_rows(W13, "w13") with N."""
+def gateup_blocked(Xb, W13, row_major_out=False):
+    """Gate/up of a Blocked X: returns a Blocked H, or a row-major tensor with row_major_out. W13: row-major tensor
+    or a Blocked from block_rows(W13, "w13")."""
     import torch
     wb = isinstance(W13, Blocked)
     N = W13.rows if wb else W13.shape[0]
     like = Xb.buf
-    Hb = Blocked(torch.empty(max(lib().fsw_blocked_bytes(Xb.rows, N // 2), 16), dtype=torch.uint8, device=like.device),
-                 Xb.rows, N // 2, Xb.dtype)
+    if row_major_out:
+        H = torch.empty((Xb.rows, N // 2), dtype=Xb.dtype, device=like.device)
+        ldh = max(N // 2, 1)
+    else:
+        H = Blocked(torch.empty(max(lib().fsw_blocked_bytes(Xb.rows, N // 2), 16), dtype=torch.uint8,
+                                device=like.device), Xb.rows, N // 2, Xb.dtype)
+        ldh = 0
     code = BF16 if Xb.dtype == torch.bfloat16 else FP16
     with torch.cuda.device(like.device):
         check(lib().fsw_gateup_blocked(code, Xb.rows, N, Xb.k, Xb.data_ptr(), W13.data_ptr(), 0 if wb else _ld(W13),
-                                       1 if wb else 0, Hb.data_ptr(), _stream(like)))
-    return Hb
+                                       1 if wb else 0, H.data_ptr(), ldh, _stream(like)))
+    return H
 
 
 def down_blocked(Hb, W2, out=None):

@@ -125,12 +125,20 @@ FSW_API int fsw_prepack_w13(int dtype, int64_t N, int64_t K, const void* W13, in
                             void* stream);
 FSW_API int fsw_prepack_w2(int dtype, int64_t D, int64_t FF, const void* W2, int64_t ldw2, void* dst_blocked,
                            void* stream);
-/* H_blocked[M, N/2] = gate/up of X_blocked[M, K]; W13 row-major (w_blocked = 0, ldw) or from fsw_prepack_w13 (1). */
+/* H[M, N/2] = gate/up of X_blocked[M, K]; W13 row-major (w_blocked = 0, ldw) or from fsw_prepack_w13 (1); H is
+ * written blocked when ldh == 0 (for fsw_down_blocked), else row-major with row stride ldh. */
 FSW_API int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* X_blocked, const void* W13,
-                               int64_t ldw, int w_blocked, void* H_blocked, void* stream);
+                               int64_t ldw, int w_blocked, void* H, int64_t ldh, void* stream);
 /* Y[M, D] (row-major, ldy) = H_blocked[M, FF] @ W2^T; W2 row-major (0, ldw2) or from fsw_prepack_w2 (1). */
 FSW_API int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* H_blocked, const void* W2,
                              int64_t ldw2, int w_blocked, void* Y, int64_t ldy, void* stream);
+
+/* fsw_gateup with optional scratch (same arguments, same result): with at least fsw_gateup_workspace_bytes() of
+ * 16-byte aligned scratch the large-tile regime re-blocks X into it first; with none (or for other shapes, where
+ * the query returns 0) it is fsw_gateup. */
+FSW_API size_t fsw_gateup_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K);
+FSW_API int fsw_gateup_ws(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13,
+                          int64_t ldw, void* H, int64_t ldh, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The hipError_t (as int) of the most recent failed launch on the calling thread, 0 if none. */
 FSW_API int fsw_last_hip_error(void);

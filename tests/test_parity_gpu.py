@@ -472,7 +472,10 @@ def test_blocked_kernels_against_oracle(capi, dtype, prepacked):
         Y = capi.down_blocked(Hb, W2)
         assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype, "blocked Y %s" % ((M, d, ff),))
         oracle.assert_parity(Y, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64), "blocked mlp %s" % ((M, d, ff),))
-        # same bits as the row-major kernels up to the fp32 summation order of the K loop (identical here: same kernel)
+        # row-major H straight from the blocked X: the same bits as the blocked H
+        Hrm = capi.gateup_blocked(Xb, W13, row_major_out=True)
+        assert torch.equal(Hrm, H)
+        # against the row-major kernels: the same products, summed in the same K order by the same kernel
         H2 = capi.gateup(g["X"], g["W13"])
         assert (H.float() - H2.float()).abs().max().item() <= 2 * ulp_rel(dtype) * 2 * H2.float().abs().max().item() + 1e-3
 
