@@ -107,6 +107,10 @@ int fsw_set_variant(int family, int variant) {
     fsw::set_raster_group(variant);
     return FSW_OK;
   }
+  if (family == 3) {  // tuning knob: kernel behind the blocked entry points when the weights are row-major
+    fsw::set_pair_ring(variant != 0);
+    return FSW_OK;
+  }
   if (family < 0 || family > 1) return FSW_E_VARIANT;
   if (variant >= 0 && variant != VARIANT_SKINNY && variant != VARIANT_DECODE_STREAM &&
       !(family == 0 && variant == VARIANT_DECODE_FUSED) &&

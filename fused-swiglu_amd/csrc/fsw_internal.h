@@ -35,6 +35,7 @@ struct TiledVariant {
   int bp, bq;        // workgroup tile: weight rows x activation rows
   int threads;
 };
+void set_pair_ring(int on);    // blocked entry points with row-major weights: pair ring (default) or plain ring
 void set_raster_group(int g);  // activation-row tiles per raster band; 0 restores the per-kernel default
 int tiled_variant_count();
 const TiledVariant& tiled_variant(int variant);

@@ -768,6 +768,256 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
   }
 }
 
+// ---- pair ring: row-major weights in whole cache lines, blocked activations ----------------------------------
+// 256 x 256 tile, 4 waves of 128 x 128, K tiles of 32 as in tiled_ring_kernel, for a ROW-MAJOR weight operand and
+// a panel-blocked activation operand. A row-major operand read 32 K elements at a time yields 64-byte requests,
+// half a cache line each; here the weight operand is fetched in K PAIRS (64 elements = one 128-byte line per row)
+// into a ring of three 32 KB pair slots, half a pair per iteration, while the activations keep a ring of four
+// 16 KB stages. A pair is issued four to three iterations before its first tile is multiplied, an activation tile
+// three iterations before. The slot/stage pattern repeats every 12 K tiles (lcm of 6 and 4), so the loop is unrolled
+// twelvefold with every LDS address a compile-time constant. 160 KB of LDS.
+// LDS layouts: pair slot = [256 rows][128 B], chunk c of row r at position c ^ ((r >> 1) & 7); activation stage =
+// [256 rows][64 B], chunk c at c ^ ((r >> 2) & 3) (both conflict-free for the operand reads, see the kernels above).
+template <class E, bool GATED, bool KTAIL, bool OBLK>
+__global__ void __launch_bounds__(256)
+tiled_pair_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
+  constexpr int WP = 2, WQ = 2, FP = 4, FQ = 4;
+  constexpr int BP = 256, BQ = 256;
+  constexpr int PSLOT = BP * 128, QSTAGE = BQ * 64;
+  constexpr int LPH = 4;  // weight copy instructions per wave per HALF pair (8 rows x 128 B each)
+  constexpr int LQ = 4;   // activation copy instructions per wave per K tile (16 rows x 64 B each)
+  constexpr int NL = LPH + LQ;
+  static_assert(!OBLK || GATED, "only H is ever written blocked");
+
+  __shared__ __align__(1024) unsigned char ps0[PSLOT];
+  __shared__ __align__(1024) unsigned char ps1[PSLOT];
+  __shared__ __align__(1024) unsigned char ps2[PSLOT];
+  __shared__ __align__(1024) unsigned char qs0[QSTAGE];
+  __shared__ __align__(1024) unsigned char qs1[QSTAGE];
+  __shared__ __align__(1024) unsigned char qs2[QSTAGE];
+  __shared__ __align__(1024) unsigned char qs3[QSTAGE];
+  unsigned char* const ps[3] = {ps0, ps1, ps2};
+  unsigned char* const qs[4] = {qs0, qs1, qs2, qs3};
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wq = wave % WQ;
+  const int wp = wave / WQ;
+  const int l32 = lane & 31;
+  const int hi = lane >> 5;
+
+  int tp, tq;
+  tile_coords(blockIdx.x, tiles_p, tiles_q, group, tp, tq);
+  const int p0 = tp * BP;
+  const int q0 = tq * BQ;
+  const int nkt = (a.k + 31) / 32;
+  const int npair = (nkt + 1) / 2;
+
+  // weight copy: lane -> chunk position pcp of row rbp (+ 32 j), fetches logical chunk lcp of the 128-byte line
+  const int pcp = t & 7;
+  const int rbp = t >> 3;
+  const int lcp = pcp ^ ((rbp >> 1) & 7);
+  const unsigned char* pbase = (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
+  const __amdgpu_buffer_rsrc_t prs = make_rsrc(pbase, ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
+  unsigned poff[2 * LPH];
+#pragma unroll
+  for (int j = 0; j < 2 * LPH; ++j) {
+    const int r = rbp + j * 32;
+    const int grow = GATED ? (r < BP / 2 ? 2 * r : 2 * (r - BP / 2) + 1) : r;
+    poff[j] = (unsigned)grow * (unsigned)a.ldp * 2u + (unsigned)lcp * 16u;
+  }
+  // activation copy from the blocked panel: lane -> chunk position pcq of row rbq (+ 64 j)
+  const int pcq = t & 3;
+  const int rbq = t >> 2;
+  const int lcq = pcq ^ ((rbq >> 2) & 3);
+  const unsigned char* qbase = (const unsigned char*)a.Q + (long long)tq * nkt * QSTAGE;
+  const __amdgpu_buffer_rsrc_t qrs = make_rsrc(qbase, (long long)nkt * QSTAGE);
+  unsigned qoff[LQ];
+#pragma unroll
+  for (int j = 0; j < LQ; ++j) qoff[j] = (unsigned)(rbq + j * 64) * 64u + (unsigned)lcq * 16u;
+
+  // operand fragment reads
+  const unsigned rd_p = (unsigned)((GATED ? wp * (FP / 2) * 32 : wp * FP * 32) + l32) * 128u;
+  const unsigned rd_q = (unsigned)(wq * FQ * 32 + l32) * 64u;
+  unsigned xp[2][2], xq[2];  // [half of the pair][K step] / [K step]
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    xq[ks] = (unsigned)((((ks << 1) | hi) ^ ((l32 >> 2) & 3)) * 16);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) xp[h][ks] = (unsigned)((((h << 2) | (ks << 1) | hi) ^ ((l32 >> 1) & 7)) * 16);
+  }
+  auto p_frag_off = [](int f) -> unsigned {
+    if (GATED) return (unsigned)((f < FP / 2 ? f * 32 : BP / 2 + (f - FP / 2) * 32) * 128);
+    return (unsigned)(f * 32 * 128);
+  };
+
+  f32x16 acc[FP][FQ];
+#pragma unroll
+  for (int f = 0; f < FP; ++f)
+#pragma unroll
+    for (int g = 0; g < FQ; ++g)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[f][g][i] = 0.0f;
+
+  // copy instruction idx of iteration kt: 0..3 = half (kt & 1) of weight pair (kt >> 1) + 2, 4..7 = activation tile
+  // kt + 3. Past the end both re-read the last pair / tile (never consumed).
+  auto dma = [&](int kt, unsigned char* pslot, unsigned char* qstage, auto lo_c, auto hi_c) {
+    constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
+    const int pair = (kt >> 1) + 2 < npair ? (kt >> 1) + 2 : npair - 1;
+    const int half = kt & 1;
+    const int qt = kt + 3 < nkt ? kt + 3 : nkt - 1;
+    const bool in = !KTAIL || (pair * 64 + lcp * 8) < a.k;
+#pragma unroll
+    for (int i = LO; i < HI; ++i) {
+      if (i < LPH) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + (half * LPH + i) * 32 * 128 + wave * 1024), 16,
+                                                 (int)(in ? poff[half * LPH + i] : OOB_OFFSET), pair * 128, 0, 0);
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(qstage + (i - LPH) * 64 * 64 + wave * 1024), 16,
+                                                 (int)qoff[i - LPH], qt * QSTAGE, 0, 0);
+      }
+    }
+  };
+  // prologue copies: a whole weight pair / one activation tile
+  auto dma_pair = [&](int pair_, unsigned char* pslot, int j_lo, int j_hi) {
+    const int pair = pair_ < npair ? pair_ : npair - 1;
+    const bool in = !KTAIL || (pair * 64 + lcp * 8) < a.k;
+#pragma unroll
+    for (int j = 0; j < 2 * LPH; ++j)
+      if (j >= j_lo && j < j_hi)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + j * 32 * 128 + wave * 1024), 16,
+                                                 (int)(in ? poff[j] : OOB_OFFSET), pair * 128, 0, 0);
+  };
+  auto dma_q = [&](int qt_, unsigned char* qstage) {
+    const int qt = qt_ < nkt ? qt_ : nkt - 1;
+#pragma unroll
+    for (int j = 0; j < LQ; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(qstage + j * 64 * 64 + wave * 1024), 16, (int)qoff[j],
+                                               qt * QSTAGE, 0, 0);
+  };
+
+  u32x4 pf[2][FP], qf[2][FQ];
+  auto f_read = [&](int fb, const unsigned char* pslot, int half, const unsigned char* qstage, int ks) {
+    pf[fb][0] = *(const u32x4*)(pslot + rd_p + p_frag_off(0) + xp[half][ks]);
+#pragma unroll
+    for (int g = 0; g < FQ; ++g) qf[fb][g] = *(const u32x4*)(qstage + rd_q + g * 32 * 64 + xq[ks]);
+#pragma unroll
+    for (int f = 1; f < FP; ++f) pf[fb][f] = *(const u32x4*)(pslot + rd_p + p_frag_off(f) + xp[half][ks]);
+  };
+  auto mma = [&](int fb, int f_lo, int f_hi) {
+#pragma unroll
+    for (int f = f_lo; f < f_hi; ++f)
+#pragma unroll
+      for (int g = 0; g < FQ; ++g) acc[f][g] = E::mfma32(pf[fb][f], qf[fb][g], acc[f][g]);
+  };
+
+  constexpr int HF = FP / 2;
+  constexpr int DA = NL / 2, DB = (NL - DA) / 2, DC = NL - DA - DB;
+  using C0 = std::integral_constant<int, 0>;
+  using CA = std::integral_constant<int, DA>;
+  using CB = std::integral_constant<int, DA + DB>;
+  using CN = std::integral_constant<int, NL>;
+  // at the barrier of iteration kt everything issued up to iteration kt - 2 has landed (tile kt + 1 and its weight
+  // pair among it); the copies of iteration kt - 1 and parts A and B of this one stay in flight
+  constexpr int VM = NL + DA + DB;
+  constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
+
+  // iteration j (mod 12) of the unrolled loop, K tile kt = base + j
+  auto iteration = [&](auto j_c, int kt) {
+    constexpr int J = decltype(j_c)::value;
+    unsigned char* const p_cur = ps[(J >> 1) % 3];
+    unsigned char* const p_nxt = ps[((J + 1) >> 1) % 3];
+    unsigned char* const p_fill = ps[((J >> 1) + 2) % 3];
+    unsigned char* const q_cur = qs[J & 3];
+    unsigned char* const q_nxt = qs[(J + 1) & 3];
+    unsigned char* const q_fill = qs[(J + 3) & 3];
+    dma(kt, p_fill, q_fill, C0{}, CA{});
+    f_read(1, p_cur, J & 1, q_cur, 1);
+    mma(0, 0, FP);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+    }
+    dma(kt, p_fill, q_fill, CA{}, CB{});
+    mma(1, 0, HF);
+#pragma unroll
+    for (int i = 0; i < DB; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, (HF * FQ) / DB, 0);
+      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+    }
+    asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(WAIT_IMM) : "memory");
+    f_read(0, p_nxt, (J + 1) & 1, q_nxt, 0);
+    dma(kt, p_fill, q_fill, CB{}, CN{});
+    mma(1, HF, FP);
+    constexpr int MC = (FP - HF) * FQ;
+#pragma unroll
+    for (int jj = 0; jj < DC; ++jj) {
+#pragma unroll
+      for (int i = 0; i < MC / DC; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, (FP + FQ + MC - 1) / MC, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+    }
+  };
+
+  if (nkt > 0) {
+    // fill in the order the loop would have issued it: [pair 0, tile 0] [pair 1 first half, tile 1] [pair 1 second
+    // half, tile 2]; then pair 0 and tile 0 have landed when 16 copies are still in flight
+    dma_pair(0, ps0, 0, 2 * LPH);
+    dma_q(0, qs0);
+    dma_pair(1, ps1, 0, LPH);
+    dma_q(1, qs1);
+    dma_pair(1, ps1, LPH, 2 * LPH);
+    dma_q(2, qs2);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NL) : "memory");
+    f_read(0, ps0, 0, qs0, 0);
+  }
+  int kt = 0;
+  for (; kt + 11 < nkt; kt += 12) {
+    iteration(std::integral_constant<int, 0>{}, kt);
+    iteration(std::integral_constant<int, 1>{}, kt + 1);
+    iteration(std::integral_constant<int, 2>{}, kt + 2);
+    iteration(std::integral_constant<int, 3>{}, kt + 3);
+    iteration(std::integral_constant<int, 4>{}, kt + 4);
+    iteration(std::integral_constant<int, 5>{}, kt + 5);
+    iteration(std::integral_constant<int, 6>{}, kt + 6);
+    iteration(std::integral_constant<int, 7>{}, kt + 7);
+    iteration(std::integral_constant<int, 8>{}, kt + 8);
+    iteration(std::integral_constant<int, 9>{}, kt + 9);
+    iteration(std::integral_constant<int, 10>{}, kt + 10);
+    iteration(std::integral_constant<int, 11>{}, kt + 11);
+  }
+#define FSW_PAIR_TAIL(J)                                     \
+  if (kt < nkt) {                                            \
+    iteration(std::integral_constant<int, J>{}, kt);         \
+    ++kt;                                                    \
+  }
+  FSW_PAIR_TAIL(0)
+  FSW_PAIR_TAIL(1)
+  FSW_PAIR_TAIL(2)
+  FSW_PAIR_TAIL(3)
+  FSW_PAIR_TAIL(4)
+  FSW_PAIR_TAIL(5)
+  FSW_PAIR_TAIL(6)
+  FSW_PAIR_TAIL(7)
+  FSW_PAIR_TAIL(8)
+  FSW_PAIR_TAIL(9)
+  FSW_PAIR_TAIL(10)
+#undef FSW_PAIR_TAIL
+
+  if constexpr (OBLK) {
+    store_tile_blocked<E, WP, WQ, FP, FQ>(acc, a, tp, tq, wp, wq, l32, hi);
+  } else {
+    store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
+  }
+}
+
 // ---- row-major -> panel-blocked copy ---------------------------------------------------------------------------
 // dst block (panel, kt) = [256 rows][64 bytes]: rows 256 panel .. 256 panel + 255 of src, K elements 32 kt .. 32 kt + 31;
 // rows past `rows` and elements past `k` are written as zeros. A workgroup copies four K tiles of one panel: reads
@@ -817,6 +1067,7 @@ const TiledVariant kVariants[] = {
 };
 
 int g_raster_group = 0;  // 0 = per-launch default
+int g_pair_ring = 1;     // row-major weights of the blocked entry points: pair ring (1) or plain ring (0)
 
 // Activation-row tiles per raster band. Measured on the headline shapes: the gate/up product (many weight
 // panels, 4096-deep K) prefers 4, the down product (few weight panels, 14336-deep K) prefers 2.
@@ -885,8 +1136,30 @@ hipError_t launch_ring_layout(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Q blocked, P row-major: the pair ring (FSW_PAIR_RING) or the plain ring with LAYOUT 1 / 3
+template <class E, bool GATED, bool OBLK>
+hipError_t launch_pair(const GemmArgs& a, hipStream_t stream) {
+  const int tiles_p = (a.np + 255) / 256;
+  const int tiles_q = (a.nq + 255) / 256;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
+  if (a.k % 64 == 0) {
+    hipLaunchKernelGGL((tiled_pair_kernel<E, GATED, false, OBLK>), grid, block, 0, stream, a, tiles_p, tiles_q,
+                       raster_group(GATED));
+  } else {
+    hipLaunchKernelGGL((tiled_pair_kernel<E, GATED, true, OBLK>), grid, block, 0, stream, a, tiles_p, tiles_q,
+                       raster_group(GATED));
+  }
+  return hipGetLastError();
+}
+
 template <class E>
 hipError_t launch_blocked_typed(bool gated, const GemmArgs& a, hipStream_t stream) {
+  if (g_pair_ring) {
+    if (gated && a.layout == 1) return launch_pair<E, true, false>(a, stream);
+    if (gated && a.layout == 3) return launch_pair<E, true, true>(a, stream);
+    if (!gated && a.layout == 1) return launch_pair<E, false, false>(a, stream);
+  }
   if (gated) {
     if (a.layout == 1) return launch_ring_layout<E, true, 5, 1>(a, stream);
     if (a.layout == 3) return launch_ring_layout<E, true, 5, 3>(a, stream);
@@ -992,6 +1265,7 @@ hipError_t launch_block_rows(const void* src, long long ld, int rows, int k, voi
 }
 
 void set_raster_group(int g) { g_raster_group = g > 0 ? g : 0; }
+void set_pair_ring(int on) { g_pair_ring = on ? 1 : 0; }
 int tiled_variant_count() { return (int)(sizeof(kVariants) / sizeof(kVariants[0])); }
 const TiledVariant& tiled_variant(int variant) { return kVariants[variant]; }
 
