@@ -376,7 +376,9 @@ static size_t h_bytes(int64_t M, int64_t FF) {
 size_t fsw_mlp_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
   if (M <= 0 || D <= 0 || FF <= 0) return 0;
   if (blocked_regime(M, D, FF)) return (size_t)fsw::blocked_bytes(M, FF) + (size_t)fsw::blocked_bytes(M, D);
-  return h_bytes(M, FF) + fsw_down_workspace_bytes(dtype, M, D, FF);
+  // otherwise [H row-major][split-K scratch of the down projection][X blocked, when gate/up alone runs large tiles]
+  return h_bytes(M, FF) + ((fsw_down_workspace_bytes(dtype, M, D, FF) + 255) & ~(size_t)255) +
+         fsw_gateup_workspace_bytes(dtype, M, 2 * FF, D);
 }
 
 int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t ldx, const void* W13, int64_t ldw13,
@@ -426,10 +428,12 @@ int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t 
     if (rc != FSW_OK) return rc;
     return fsw_down_blocked(dtype, M, D, FF, Hb, W2, ldw2, 0, Y, ldy, stream);
   }
-  rc = fsw_gateup(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF, stream);
-  if (rc != FSW_OK) return rc;
   unsigned char* ws2 = (unsigned char*)workspace + h_bytes(M, FF);
-  return fsw_down(dtype, M, D, FF, Hbuf, FF, W2, ldw2, Y, ldy, ws2, workspace_bytes - h_bytes(M, FF), stream);
+  const size_t down_ws = (fsw_down_workspace_bytes(dtype, M, D, FF) + 255) & ~(size_t)255;
+  rc = fsw_gateup_ws(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF, ws2 + down_ws,
+                     fsw_gateup_workspace_bytes(dtype, M, 2 * FF, D), stream);
+  if (rc != FSW_OK) return rc;
+  return fsw_down(dtype, M, D, FF, Hbuf, FF, W2, ldw2, Y, ldy, ws2, down_ws, stream);
 }
 
 }  // extern "C"
