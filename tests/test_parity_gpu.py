@@ -480,6 +480,31 @@ def test_blocked_kernels_against_oracle(capi, dtype, prepacked):
         assert (H.float() - H2.float()).abs().max().item() <= 2 * ulp_rel(dtype) * 2 * H2.float().abs().max().item() + 1e-3
 
 
+def test_blocked_kernels_take_strided_row_major_operands(capi):
+    """Row strides larger than the row (column slices of wider tensors) for X into fsw_block_rows, for the
+    row-major W13 / W2 of the pair-ring kernels and for Y; also the other kernel behind the blocked entry points
+    (plain ring, fsw_set_variant(3, 0)) must give the same bits."""
+    M, d, ff = 300, 1096, 520
+    dtype = torch.bfloat16
+    inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=123, x_scale=0.5)
+    wide = lambda t, extra: torch.cat([t, torch.full((t.shape[0], extra), float("nan"), dtype=t.dtype)], dim=1).to(DEV)[:, : t.shape[1]]
+    X, W13, W2 = wide(inp["X"], 24), wide(inp["W13"], 8), wide(inp["W2"], 40)
+    assert X.stride(0) == d + 24 and W13.stride(0) == d + 8 and W2.stride(0) == ff + 40
+    Xb = capi.block_rows(X)
+    Hb = capi.gateup_blocked(Xb, W13)
+    Ybig = torch.full((M, d + 16), float("nan"), dtype=dtype, device=DEV)
+    Y = capi.down_blocked(Hb, W2, out=Ybig[:, :d])
+    oracle.assert_parity(Y, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64), "blocked, strided operands")
+    assert torch.isnan(Ybig[:, d:]).all()
+    try:
+        capi.set_variant(3, 0)
+        Hb2 = capi.gateup_blocked(Xb, W13)
+        Y2 = capi.down_blocked(Hb2, W2)
+    finally:
+        capi.set_variant(3, 1)
+    assert torch.equal(capi.unblock(Hb2), capi.unblock(Hb)) and torch.equal(Y2, Y)
+
+
 def test_mlp_large_tile_regime_uses_blocked_path(capi):
     """For M > 64 with both projections on 256 x 256 tiles fsw_mlp re-blocks X into the workspace and keeps H blocked;
     the result agrees with the separate row-major entry points and with the oracle, and the workspace query covers
