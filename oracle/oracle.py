@@ -28,7 +28,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "_build", "liboracle.so")
 
 BF16, FP16 = 0, 1
-# north-star gates: max |out - ref| and mean|out - ref| / mean|ref|
+# tolerance gates: max |out - ref| and mean|out - ref| / mean|ref|
 MAX_ABS_TOL = 2e-2
 MEAN_REL_TOL = 5e-3
 
