@@ -775,7 +775,8 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
 // into a ring of three 32 KB pair slots, half a pair per iteration, while the activations keep a ring of four
 // 16 KB stages. A pair is issued four to three iterations before its first tile is multiplied, an activation tile
 // three iterations before. The slot/stage pattern repeats every 12 K tiles (lcm of 6 and 4), so the loop is unrolled
-// twelvefold with every LDS address a compile-time constant. 160 KB of LDS.
+// twelvefold with every LDS address a compile-time constant. 160 KB of LDS. The workgroup barrier sits between the two
+// K steps of a tile and the instruction order of each half is written out by hand (see half_iteration).
 // LDS layouts: pair slot = [256 rows][128 B], chunk c of row r at position c ^ ((r >> 1) & 7); activation stage =
 // [256 rows][64 B], chunk c at c ^ ((r >> 2) & 3) (both conflict-free for the operand reads, see the kernels above).
 template <class E, bool GATED, bool KTAIL, bool OBLK>
@@ -898,31 +899,60 @@ tiled_pair_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
   };
 
   u32x4 pf[2][FP], qf[2][FQ];
-  auto f_read = [&](int fb, const unsigned char* pslot, int half, const unsigned char* qstage, int ks) {
-    pf[fb][0] = *(const u32x4*)(pslot + rd_p + p_frag_off(0) + xp[half][ks]);
-#pragma unroll
-    for (int g = 0; g < FQ; ++g) qf[fb][g] = *(const u32x4*)(qstage + rd_q + g * 32 * 64 + xq[ks]);
-#pragma unroll
-    for (int f = 1; f < FP; ++f) pf[fb][f] = *(const u32x4*)(pslot + rd_p + p_frag_off(f) + xp[half][ks]);
-  };
-  auto mma = [&](int fb, int f_lo, int f_hi) {
-#pragma unroll
-    for (int f = f_lo; f < f_hi; ++f)
-#pragma unroll
-      for (int g = 0; g < FQ; ++g) acc[f][g] = E::mfma32(pf[fb][f], qf[fb][g], acc[f][g]);
-  };
-
-  constexpr int HF = FP / 2;
-  constexpr int DA = NL / 2, DB = (NL - DA) / 2, DC = NL - DA - DB;
   using C0 = std::integral_constant<int, 0>;
-  using CA = std::integral_constant<int, DA>;
-  using CB = std::integral_constant<int, DA + DB>;
-  using CN = std::integral_constant<int, NL>;
-  // at the barrier of iteration kt everything issued up to iteration kt - 2 has landed (tile kt + 1 and its weight
-  // pair among it); the copies of iteration kt - 1 and parts A and B of this one stay in flight
-  constexpr int VM = NL + DA + DB;
+  using CH = std::integral_constant<int, LPH>;
+  // The barrier sits in the middle of the iteration, between the two K steps. At the barrier of iteration kt
+  // everything issued up to iteration kt - 2 has landed (tile kt + 1 and its weight pair among it); the copies of
+  // iteration kt - 1 and the first half of this one stay in flight. lgkmcnt(0): this wave's reads of tile kt are
+  // complete (the last one was issued eight MFMAs earlier), so its stage may be refilled from the next iteration on.
+  constexpr int VM = NL + LPH;
   constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
 
+  // One fragment read / one MFMA by index, for the hand-ordered halves below. Read order: P fragment 0, the FQ
+  // activation fragments, then P fragments 1 .. FP-1: the order the MFMAs (f major, g minor) first need them.
+  auto read_one = [&](int fb, int idx, const unsigned char* pslot, int half, const unsigned char* qstage, int ks) {
+    if (idx == 0) {
+      pf[fb][0] = *(const u32x4*)(pslot + rd_p + p_frag_off(0) + xp[half][ks]);
+    } else if (idx <= FQ) {
+      qf[fb][idx - 1] = *(const u32x4*)(qstage + rd_q + (idx - 1) * 32 * 64 + xq[ks]);
+    } else {
+      pf[fb][idx - FQ] = *(const u32x4*)(pslot + rd_p + p_frag_off(idx - FQ) + xp[half][ks]);
+    }
+  };
+  auto mma_one = [&](int fb, int i) {
+    acc[i / FQ][i % FQ] = E::mfma32(pf[fb][i / FQ], qf[fb][i % FQ], acc[i / FQ][i % FQ]);
+  };
+  // Half an iteration: the 16 MFMAs of K step `ks_mma` with, between them, first the 8 fragment reads of the
+  // following K step (one per MFMA) and then 4 copies (one per two MFMAs): at most one other instruction between two
+  // MFMAs, in exactly this order (the scheduler is fenced after every group).
+  auto half_iteration = [&](int fb_mma, int fb_rd, const unsigned char* pslot_rd, int half_rd,
+                            const unsigned char* qstage_rd, int ks_rd, int kt, unsigned char* p_fill,
+                            unsigned char* q_fill, auto lo_c) {
+    constexpr int LO = decltype(lo_c)::value;
+    static_assert(FP + FQ + 2 * LPH == FP * FQ && LPH == 4, "16 MFMAs = 8 read slots + 4 copy slots of two");
+#pragma unroll
+    for (int i = 0; i < FP + FQ; ++i) {
+      mma_one(fb_mma, i);
+      read_one(fb_rd, i, pslot_rd, half_rd, qstage_rd, ks_rd);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    mma_one(fb_mma, FP + FQ + 0);
+    mma_one(fb_mma, FP + FQ + 1);
+    dma(kt, p_fill, q_fill, std::integral_constant<int, LO>{}, std::integral_constant<int, LO + 1>{});
+    __builtin_amdgcn_sched_barrier(0);
+    mma_one(fb_mma, FP + FQ + 2);
+    mma_one(fb_mma, FP + FQ + 3);
+    dma(kt, p_fill, q_fill, std::integral_constant<int, LO + 1>{}, std::integral_constant<int, LO + 2>{});
+    __builtin_amdgcn_sched_barrier(0);
+    mma_one(fb_mma, FP + FQ + 4);
+    mma_one(fb_mma, FP + FQ + 5);
+    dma(kt, p_fill, q_fill, std::integral_constant<int, LO + 2>{}, std::integral_constant<int, LO + 3>{});
+    __builtin_amdgcn_sched_barrier(0);
+    mma_one(fb_mma, FP + FQ + 6);
+    mma_one(fb_mma, FP + FQ + 7);
+    dma(kt, p_fill, q_fill, std::integral_constant<int, LO + 3>{}, std::integral_constant<int, LO + 4>{});
+    __builtin_amdgcn_sched_barrier(0);
+  };
   // iteration j (mod 12) of the unrolled loop, K tile kt = base + j
   auto iteration = [&](auto j_c, int kt) {
     constexpr int J = decltype(j_c)::value;
@@ -932,38 +962,9 @@ tiled_pair_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
     unsigned char* const q_cur = qs[J & 3];
     unsigned char* const q_nxt = qs[(J + 1) & 3];
     unsigned char* const q_fill = qs[(J + 3) & 3];
-    dma(kt, p_fill, q_fill, C0{}, CA{});
-    f_read(1, p_cur, J & 1, q_cur, 1);
-    mma(0, 0, FP);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
-    }
-    dma(kt, p_fill, q_fill, CA{}, CB{});
-    mma(1, 0, HF);
-#pragma unroll
-    for (int i = 0; i < DB; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, (HF * FQ) / DB, 0);
-      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
-    }
+    half_iteration(0, 1, p_cur, J & 1, q_cur, 1, kt, p_fill, q_fill, C0{});
     asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(WAIT_IMM) : "memory");
-    f_read(0, p_nxt, (J + 1) & 1, q_nxt, 0);
-    dma(kt, p_fill, q_fill, CB{}, CN{});
-    mma(1, HF, FP);
-    constexpr int MC = (FP - HF) * FQ;
-#pragma unroll
-    for (int jj = 0; jj < DC; ++jj) {
-#pragma unroll
-      for (int i = 0; i < MC / DC; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x100, (FP + FQ + MC - 1) / MC, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
-    }
+    half_iteration(1, 0, p_nxt, (J + 1) & 1, q_nxt, 0, kt, p_fill, q_fill, CH{});
   };
 
   if (nkt > 0) {
@@ -976,7 +977,8 @@ tiled_pair_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
     dma_pair(1, ps1, LPH, 2 * LPH);
     dma_q(2, qs2);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NL) : "memory");
-    f_read(0, ps0, 0, qs0, 0);
+#pragma unroll
+    for (int i = 0; i < FP + FQ; ++i) read_one(0, i, ps0, 0, qs0, 0);
   }
   int kt = 0;
   for (; kt + 11 < nkt; kt += 12) {
