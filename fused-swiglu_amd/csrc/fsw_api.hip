@@ -352,6 +352,11 @@ size_t fsw_gateup_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K) {
   (void)dtype;
   if (M <= 64 || N <= 0 || K <= 0 || M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return 0;
   if (g_forced_variant[0] >= 0 || pick_tiled(0, M, N) != 8) return 0;
+  // Few activation panels with a ragged last one: the re-block launch and the zero rows of the padded panel (read
+  // from memory, where the row-major kernel's out-of-range rows cost no traffic) outweigh the whole-line requests.
+  // Measured at 4096 x 28672, blocked vs row-major ring: M = 384: 145 vs 129 us, 576: 215 vs 190, 640: 216 vs 199,
+  // 896: 222 vs 211, 960: 223 vs 219; M = 512: 141 vs 147, 1024: 226 vs 241, 1152: level, 1536: 310 vs 329.
+  if (M < 1024 && M % 256 != 0) return 0;
   return (size_t)fsw::blocked_bytes(M, K);
 }
 

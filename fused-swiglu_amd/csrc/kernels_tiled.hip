@@ -1066,6 +1066,7 @@ const TiledVariant kVariants[] = {
     {"ring8w_256x256_b", 256, 256, 512},  // 8 waves, wave tile 64 x 128
     {"dma8w_256x256", 256, 256, 512},
     {"ring5_256x256", 256, 256, 256},  // five-stage ring: all 160 KB of LDS, four K tiles in flight
+    {"ring5_256x192", 256, 192, 256},  // 192 activation rows: fewer padded rows / idle CUs for some M (see pick_tiled)
 };
 
 int g_raster_group = 0;  // 0 = per-launch default
@@ -1191,6 +1192,7 @@ hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
     case 11: return launch_ring<E, GATED, 4, 4, 2, 2, 4>(a, stream);
     case 12: return launch_dma<E, GATED, 2, 4, 4, 2>(a, stream);
     case 13: return launch_ring<E, GATED, 5, 2, 2, 4, 4>(a, stream);
+    case 14: return launch_ring<E, GATED, 5, 2, 2, 4, 3>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
