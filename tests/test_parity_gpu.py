@@ -519,3 +519,30 @@ def test_mlp_large_tile_regime_uses_blocked_path(capi):
     rows = torch.arange(0, M, 37)
     oracle.assert_parity(Y[rows.to(DEV)], oracle.ref_mlp(inp["X"][rows], inp["W13"], inp["W2"], torch.float64), "mlp blocked regime")
     assert (Y.float() - Y2.float()).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("shape", [(16, 512, 1024), (96, 512, 1024), (600, 1024, 520)])
+def test_forward_replays_from_a_hip_graph(capi, shape):
+    """fsw_mlp enqueues kernels only (no allocation, no synchronisation, no memset), so a caller can capture it into a
+    HIP graph. Every replay — with eager work and synchronisations of the program in between, and with new contents
+    in the input buffer — must reproduce the eager result bit for bit. Decode, mid and large-tile regimes."""
+    M, d, ff = shape
+    inp = fsw_weights.make_inputs(M, d, ff, torch.bfloat16, seed=123, x_scale=0.5)
+    g = to_dev(inp)
+    X = g["X"].clone()
+    Y = torch.empty(M, d, dtype=torch.bfloat16, device=DEV)
+    ws = capi.mlp_workspace(X, ff)
+    capi.mlp(X, g["W13"], g["W2"], out=Y, workspace=ws)  # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        capi.mlp(X, g["W13"], g["W2"], out=Y, workspace=ws)
+    for rep in range(3):
+        X.copy_(g["X"] * (1.0 + 0.25 * rep))
+        eager = capi.mlp(X, g["W13"], g["W2"])
+        torch.cuda.synchronize()
+        Y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Y, eager), "replay %d differs from the eager forward" % rep
+    oracle.assert_parity(Y, oracle.ref_mlp(X.cpu(), inp["W13"], inp["W2"], torch.float64), "graph replay")
