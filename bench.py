@@ -197,7 +197,7 @@ def main():
                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "algorithmic_bytes": all_bytes,
                     "avg_kernel_ms": round(gu_ms, 5)}
     else:
-        kname = "pair_256x256, X and H panel-blocked" if blocked else capi.variant_name(0, 0, M, 2 * ff, d)
+        kname = "pair16_256x256 (v_mfma_f32_16x16x32), X and H panel-blocked" if blocked else capi.variant_name(0, 0, M, 2 * ff, d)
         roofline = {"bound": "mfma", "kernel": kname + " (gate/up)",
                     "achieved": round(gu_tflops, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(gu_tflops / MFMA_PEAK_TFLOPS, 4),

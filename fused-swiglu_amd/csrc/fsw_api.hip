@@ -108,7 +108,7 @@ int fsw_set_variant(int family, int variant) {
     return FSW_OK;
   }
   if (family == 3) {  // tuning knob: kernel behind the blocked entry points when the weights are row-major
-    fsw::set_pair_ring(variant != 0);
+    fsw::set_pair_ring(variant);
     return FSW_OK;
   }
   if (family < 0 || family > 1) return FSW_E_VARIANT;

@@ -24,6 +24,14 @@ struct Bf16 {
   static __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
+  // The same instruction accumulating IN PLACE in accumulation registers ("+a": destination tied to the addend).
+  // With 64 accumulator tiles live across an unrolled loop the register allocator does not always tie the builtin's
+  // result to its addend and then moves accumulators between MFMAs; written out, the tie is part of the
+  // instruction. The compiler does not see inside the statement: code that reads the accumulators with other
+  // instructions afterwards must let the last MFMA drain first (mfma_drain).
+  static __device__ __forceinline__ void mfma16_acc(f32x4& c, u32x4 a, u32x4 b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
   static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
     bf16x2 v = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(unsigned, v);
@@ -42,6 +50,9 @@ struct Fp16 {
   static __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
+  static __device__ __forceinline__ void mfma16_acc(f32x4& c, u32x4 a, u32x4 b) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
   static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
     f16x2 v = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(unsigned, v);
@@ -51,6 +62,10 @@ struct Fp16 {
     return __builtin_bit_cast(unsigned short, v);
   }
 };
+
+// Wait states between the last hand-written MFMA and the first other instruction that reads its accumulators
+// (the longest requirement listed for matrix results read by vector instructions is 18).
+__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
 
 // silu(x) = x / (1 + e^-x) (swiglu.cu:96) with v_exp_f32 (2^x) and v_rcp_f32; both are ~1 ulp fp32, far
 // below the half-precision rounding applied afterwards. x -> -inf gives x * rcp(inf) = -0, no NaN for finite x.

@@ -152,6 +152,8 @@ FSW_API int fsw_version(void);
  * persistent streaming kernel (honoured for M <= 16; automatic only for d * ff >= 2^27); family 0 variant 101
  * makes fsw_mlp run M <= 16 as one persistent launch (gate/up, device-wide barrier, down) instead of two launches.
  * family 2 sets the raster band height of the tiled kernels instead (0 = per-kernel default).
+ * family 3 picks the kernel behind the blocked entry points for row-major weights: 2 = pair ring on
+ * v_mfma_f32_16x16x32 (default), 1 = pair ring on v_mfma_f32_32x32x16, 0 = plain ring.
  * Returns FSW_E_VARIANT for unknown ids. Process-wide and not thread-safe against concurrent launches.
  */
 FSW_API int fsw_set_variant(int family, int variant);

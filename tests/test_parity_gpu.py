@@ -483,7 +483,7 @@ def test_blocked_kernels_against_oracle(capi, dtype, prepacked):
 def test_blocked_kernels_take_strided_row_major_operands(capi):
     """Row strides larger than the row (column slices of wider tensors) for X into fsw_block_rows, for the
     row-major W13 / W2 of the pair-ring kernels and for Y; also the other kernel behind the blocked entry points
-    (plain ring, fsw_set_variant(3, 0)) must give the same bits."""
+    (plain ring, fsw_set_variant(3, 0); pair ring on 32x32x16 MFMAs, (3, 1)) must give the same bits."""
     M, d, ff = 300, 1096, 520
     dtype = torch.bfloat16
     inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=123, x_scale=0.5)
@@ -496,13 +496,14 @@ def test_blocked_kernels_take_strided_row_major_operands(capi):
     Y = capi.down_blocked(Hb, W2, out=Ybig[:, :d])
     oracle.assert_parity(Y, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64), "blocked, strided operands")
     assert torch.isnan(Ybig[:, d:]).all()
-    try:
-        capi.set_variant(3, 0)
-        Hb2 = capi.gateup_blocked(Xb, W13)
-        Y2 = capi.down_blocked(Hb2, W2)
-    finally:
-        capi.set_variant(3, 1)
-    assert torch.equal(capi.unblock(Hb2), capi.unblock(Hb)) and torch.equal(Y2, Y)
+    for mode in (0, 1):  # plain ring, pair ring on 32x32x16 MFMAs; the default (2) is the pair ring on 16x16x32
+        try:
+            capi.set_variant(3, mode)
+            Hb2 = capi.gateup_blocked(Xb, W13)
+            Y2 = capi.down_blocked(Hb2, W2)
+        finally:
+            capi.set_variant(3, 2)
+        assert torch.equal(capi.unblock(Hb2), capi.unblock(Hb)) and torch.equal(Y2, Y), "mode %d" % mode
 
 
 def test_mlp_large_tile_regime_uses_blocked_path(capi):
