@@ -917,10 +917,10 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   using C0 = std::integral_constant<int, 0>;
   using CH = std::integral_constant<int, LPH>;
   // The barrier sits in the middle of the iteration. At the barrier of iteration kt everything issued up to
-  // iteration kt - 2 has landed (tile kt + 1 and its weight pair among it); the copies of iteration kt - 1 and the
-  // first half of this one stay in flight. lgkmcnt(0): this wave's reads of tile kt (issued in the second half of
+  // iteration kt - 2 has landed (tile kt + 1 and its weight pair among it); the copies of iteration kt - 1 and of
+  // this one stay in flight. lgkmcnt(0): this wave's reads of tile kt (issued in the second half of
   // iteration kt - 1) are complete, so its stage may be refilled from the next iteration on.
-  constexpr int VM = NL + LPH;
+  constexpr int VM = NL + NL;
   constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
 
   // Fragment read by index: weight block 0, the 8 activation blocks, then weight blocks 1 .. 7: the order the MFMAs
@@ -938,9 +938,10 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
     E::mfma16_acc(acc[i / NB][i % NB], fr[set][i / NB], fr[set][NB + i % NB]);
   };
   // iteration j (mod 12) of the unrolled loop, K tile kt = base + j, fragments of tile kt in register set j & 1.
-  // First half: the 32 MFMAs of weight blocks 0 .. 3 with the four weight copies between them; barrier; second half:
-  // the 32 MFMAs of weight blocks 4 .. 7 with the 16 fragment reads of tile kt + 1 (one per two MFMAs) and the four
-  // activation copies. The scheduler is fenced after every group, so this is the issue order.
+  // First half: the 32 MFMAs of weight blocks 0 .. 3 with the eight copies between them (one per four MFMAs);
+  // barrier; second half: the 32 MFMAs of weight blocks 4 .. 7 with the 16 fragment reads of tile kt + 1 (one per two
+  // MFMAs). The scheduler is fenced after every group, so this is the issue order. (A copy next to a read between two
+  // 16-cycle MFMAs — s_mov m0, the copy, the read, a wait — does not fit their shadow.)
   auto iteration = [&](auto j_c, int kt) {
     constexpr int J = decltype(j_c)::value;
     constexpr int SET = J & 1;
@@ -951,12 +952,14 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
 #define FSW_P16_GROUP(G)                                                                                      \
     mma_one(SET, 8 * (G) + 0);                                                                                 \
     mma_one(SET, 8 * (G) + 1);                                                                                 \
-    dma(kt, p_fill, q_fill, std::integral_constant<int, (G)>{}, std::integral_constant<int, (G) + 1>{});       \
+    dma(kt, p_fill, q_fill, std::integral_constant<int, 2 * (G)>{}, std::integral_constant<int, 2 * (G) + 1>{}); \
     __builtin_amdgcn_sched_barrier(0);                                                                         \
     mma_one(SET, 8 * (G) + 2);                                                                                 \
     mma_one(SET, 8 * (G) + 3);                                                                                 \
     mma_one(SET, 8 * (G) + 4);                                                                                 \
     mma_one(SET, 8 * (G) + 5);                                                                                 \
+    dma(kt, p_fill, q_fill, std::integral_constant<int, 2 * (G) + 1>{}, std::integral_constant<int, 2 * (G) + 2>{}); \
+    __builtin_amdgcn_sched_barrier(0);                                                                         \
     mma_one(SET, 8 * (G) + 6);                                                                                 \
     mma_one(SET, 8 * (G) + 7);                                                                                 \
     __builtin_amdgcn_sched_barrier(0);
@@ -972,10 +975,6 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
       read_one(SET ^ 1, r, p_nxt, (J + 1) & 1, q_nxt);
       mma_one(SET, 4 * NB + 2 * r + 1);
       __builtin_amdgcn_sched_barrier(0);
-      if (r == 3) dma(kt, p_fill, q_fill, std::integral_constant<int, LPH>{}, std::integral_constant<int, LPH + 1>{});
-      if (r == 7) dma(kt, p_fill, q_fill, std::integral_constant<int, LPH + 1>{}, std::integral_constant<int, LPH + 2>{});
-      if (r == 11) dma(kt, p_fill, q_fill, std::integral_constant<int, LPH + 2>{}, std::integral_constant<int, LPH + 3>{});
-      if (r == 15) dma(kt, p_fill, q_fill, std::integral_constant<int, LPH + 3>{}, std::integral_constant<int, LPH + 4>{});
     }
     __builtin_amdgcn_sched_barrier(0);
   };
