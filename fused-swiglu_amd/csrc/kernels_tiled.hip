@@ -798,7 +798,10 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
 // Accumulators are a two-dimensional array indexed by constants only (a flat array made the register allocator move
 // accumulators between MFMAs).
 // [the description of the rings follows at tiled_pair_kernel]
-template <class E, bool GATED, bool KTAIL, bool OBLK>
+// PBLK: the weight operand is panel-blocked as well (prepacked; for the gated kernel in de-interleaved row order). It
+// then arrives like the activations, one 16 KB block per K tile, and keeps a ring of four 64-byte-row stages instead
+// of the pair slots (128 KB of LDS).
+template <class E, bool GATED, bool KTAIL, bool OBLK, bool PBLK = false>
 __global__ void __launch_bounds__(256)
 tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
   constexpr int WP = 2, WQ = 2;
@@ -809,15 +812,19 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   constexpr int LQ = 4;   // activation copy instructions per wave per K tile (16 rows x 64 B each)
   constexpr int NL = LPH + LQ;
   static_assert(!OBLK || GATED, "only H is ever written blocked");
+  static_assert(!PBLK || !KTAIL, "blocked operands are zero padded in K");
+  constexpr int PSTAGE = BP * 64;
+  constexpr int PBUF = PBLK ? PSTAGE : PSLOT;
 
-  __shared__ __align__(1024) unsigned char ps0[PSLOT];
-  __shared__ __align__(1024) unsigned char ps1[PSLOT];
-  __shared__ __align__(1024) unsigned char ps2[PSLOT];
+  __shared__ __align__(1024) unsigned char ps0[PBUF];
+  __shared__ __align__(1024) unsigned char ps1[PBUF];
+  __shared__ __align__(1024) unsigned char ps2[PBUF];
+  __shared__ alignas(PBLK ? 1024 : 16) unsigned char ps3[PBLK ? PSTAGE : 16];
   __shared__ __align__(1024) unsigned char qs0[QSTAGE];
   __shared__ __align__(1024) unsigned char qs1[QSTAGE];
   __shared__ __align__(1024) unsigned char qs2[QSTAGE];
   __shared__ __align__(1024) unsigned char qs3[QSTAGE];
-  unsigned char* const ps[3] = {ps0, ps1, ps2};
+  unsigned char* const ps[4] = {ps0, ps1, ps2, ps3};
   unsigned char* const qs[4] = {qs0, qs1, qs2, qs3};
 
   const int t = threadIdx.x;
@@ -839,8 +846,10 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   const int pcp = t & 7;
   const int rbp = t >> 3;
   const int lcp = pcp ^ ((rbp >> 1) & 7);
-  const unsigned char* pbase = (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
-  const __amdgpu_buffer_rsrc_t prs = make_rsrc(pbase, ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
+  const unsigned char* pbase = PBLK ? (const unsigned char*)a.P + (long long)tp * nkt * PSTAGE
+                                    : (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
+  const __amdgpu_buffer_rsrc_t prs =
+      make_rsrc(pbase, PBLK ? (long long)nkt * PSTAGE : ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
   unsigned poff[2 * LPH];
 #pragma unroll
   for (int j = 0; j < 2 * LPH; ++j) {
@@ -859,14 +868,17 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   for (int j = 0; j < LQ; ++j) qoff[j] = (unsigned)(rbq + j * 64) * 64u + (unsigned)lcq * 16u;
 
   // operand fragment of a 16-row block: lane -> row r16, 16-byte K chunk c4 of the 32-element K tile
-  const unsigned rd_p = (unsigned)((GATED ? wp * 64 : wp * 128) + r16) * 128u;
+  const unsigned rd_p = PBLK ? (unsigned)((GATED ? wp * 64 : wp * 128) + r16) * 64u +
+                                   (unsigned)((c4 ^ ((r16 >> 2) & 3)) * 16)
+                             : (unsigned)((GATED ? wp * 64 : wp * 128) + r16) * 128u;
   const unsigned rd_q = (unsigned)(wq * 128 + r16) * 64u + (unsigned)((c4 ^ ((r16 >> 2) & 3)) * 16);
   unsigned xp[2];  // [half of the pair]
 #pragma unroll
   for (int h = 0; h < 2; ++h) xp[h] = (unsigned)((((h << 2) | c4) ^ ((r16 >> 1) & 7)) * 16);
   auto p_block_off = [](int f) -> unsigned {
-    if (GATED) return (unsigned)((f < NB / 2 ? f * 16 : BP / 2 + (f - NB / 2) * 16) * 128);
-    return (unsigned)(f * 16 * 128);
+    constexpr unsigned RB = PBLK ? 64 : 128;  // bytes per weight row in LDS
+    if (GATED) return (unsigned)(f < NB / 2 ? f * 16 : BP / 2 + (f - NB / 2) * 16) * RB;
+    return (unsigned)(f * 16) * RB;
   };
 
   f32x4 acc[NB][NB];
@@ -885,7 +897,10 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
     const bool in = !KTAIL || (pair * 64 + lcp * 8) < a.k;
 #pragma unroll
     for (int i = LO; i < HI; ++i) {
-      if (i < LPH) {
+      if (i < LPH && PBLK) {  // weight tile kt + 3, copied like an activation tile
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + i * 64 * 64 + wave * 1024), 16, (int)qoff[i],
+                                                 qt * PSTAGE, 0, 0);
+      } else if (i < LPH) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + (half * LPH + i) * 32 * 128 + wave * 1024), 16,
                                                  (int)(in ? poff[half * LPH + i] : OOB_OFFSET), pair * 128, 0, 0);
       } else {
@@ -903,6 +918,13 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
       if (j >= j_lo && j < j_hi)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + j * 32 * 128 + wave * 1024), 16,
                                                  (int)(in ? poff[j] : OOB_OFFSET), pair * 128, 0, 0);
+  };
+  auto dma_pb = [&](int pt_, unsigned char* pstage) {
+    const int pt = pt_ < nkt ? pt_ : nkt - 1;
+#pragma unroll
+    for (int j = 0; j < LPH; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pstage + j * 64 * 64 + wave * 1024), 16, (int)qoff[j],
+                                               pt * PSTAGE, 0, 0);
   };
   auto dma_q = [&](int qt_, unsigned char* qstage) {
     const int qt = qt_ < nkt ? qt_ : nkt - 1;
@@ -927,11 +949,11 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   // (f major, g minor) first need them.
   auto read_one = [&](int set, int idx, const unsigned char* pslot, int half, const unsigned char* qstage) {
     if (idx == 0) {
-      fr[set][0] = *(const u32x4*)(pslot + rd_p + p_block_off(0) + xp[half]);
+      fr[set][0] = *(const u32x4*)(pslot + rd_p + p_block_off(0) + (PBLK ? 0u : xp[half]));
     } else if (idx <= NB) {
       fr[set][NB + idx - 1] = *(const u32x4*)(qstage + rd_q + (idx - 1) * 16 * 64);
     } else {
-      fr[set][idx - NB] = *(const u32x4*)(pslot + rd_p + p_block_off(idx - NB) + xp[half]);
+      fr[set][idx - NB] = *(const u32x4*)(pslot + rd_p + p_block_off(idx - NB) + (PBLK ? 0u : xp[half]));
     }
   };
   auto mma_one = [&](int set, int i) {
@@ -945,8 +967,8 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   auto iteration = [&](auto j_c, int kt) {
     constexpr int J = decltype(j_c)::value;
     constexpr int SET = J & 1;
-    unsigned char* const p_nxt = ps[((J + 1) >> 1) % 3];
-    unsigned char* const p_fill = ps[((J >> 1) + 2) % 3];
+    unsigned char* const p_nxt = PBLK ? ps[(J + 1) & 3] : ps[((J + 1) >> 1) % 3];
+    unsigned char* const p_fill = PBLK ? ps[(J + 3) & 3] : ps[((J >> 1) + 2) % 3];
     unsigned char* const q_nxt = qs[(J + 1) & 3];
     unsigned char* const q_fill = qs[(J + 3) & 3];
 #define FSW_P16_GROUP(G)                                                                                      \
@@ -982,12 +1004,21 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   if (nkt > 0) {
     // fill in the order the loop would have issued it: [pair 0, tile 0] [pair 1 first half, tile 1] [pair 1 second
     // half, tile 2]; then pair 0 and tile 0 have landed when 16 copies are still in flight
-    dma_pair(0, ps0, 0, 2 * LPH);
-    dma_q(0, qs0);
-    dma_pair(1, ps1, 0, LPH);
-    dma_q(1, qs1);
-    dma_pair(1, ps1, LPH, 2 * LPH);
-    dma_q(2, qs2);
+    if constexpr (PBLK) {
+      dma_pb(0, ps0);
+      dma_q(0, qs0);
+      dma_pb(1, ps1);
+      dma_q(1, qs1);
+      dma_pb(2, ps2);
+      dma_q(2, qs2);
+    } else {
+      dma_pair(0, ps0, 0, 2 * LPH);
+      dma_q(0, qs0);
+      dma_pair(1, ps1, 0, LPH);
+      dma_q(1, qs1);
+      dma_pair(1, ps1, LPH, 2 * LPH);
+      dma_q(2, qs2);
+    }
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NL) : "memory");
 #pragma unroll
     for (int i = 0; i < 2 * NB; ++i) read_one(0, i, ps0, 0, qs0);
@@ -1496,12 +1527,26 @@ hipError_t launch_pair16(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// both operands blocked (prepacked weights): the 16x16x32 kernel with a stage ring for the weights
+template <class E, bool GATED, bool OBLK>
+hipError_t launch_pair16_blocked(const GemmArgs& a, hipStream_t stream) {
+  const int tiles_p = (a.np + 255) / 256;
+  const int tiles_q = (a.nq + 255) / 256;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK, true>), dim3((unsigned)(tiles_p * tiles_q)), dim3(256), 0,
+                     stream, a, tiles_p, tiles_q, raster_group(GATED));
+  return hipGetLastError();
+}
+
 template <class E>
 hipError_t launch_blocked_typed(bool gated, const GemmArgs& a, hipStream_t stream) {
   if (g_pair_ring == 2) {
     if (gated && a.layout == 1) return launch_pair16<E, true, false>(a, stream);
     if (gated && a.layout == 3) return launch_pair16<E, true, true>(a, stream);
     if (!gated && a.layout == 1) return launch_pair16<E, false, false>(a, stream);
+    if (gated && a.layout == 5) return launch_pair16_blocked<E, true, false>(a, stream);
+    if (gated && a.layout == 7) return launch_pair16_blocked<E, true, true>(a, stream);
+    if (!gated && a.layout == 5) return launch_pair16_blocked<E, false, false>(a, stream);
   }
   if (g_pair_ring) {
     if (gated && a.layout == 1) return launch_pair<E, true, false>(a, stream);

@@ -77,8 +77,10 @@ FSW_API int fsw_validate_down(int dtype, int64_t M, int64_t D, int64_t FF,
                       const void* H, int64_t ldh, const void* W2, int64_t ldw2,
                       const void* Y, int64_t ldy);
 
-/* Bytes of device scratch fsw_down needs for this shape (fp32 split-K partials in the small-M regime;
- * 0 when the shape runs without scratch). No counterpart in the reference, which has no down projection. */
+/* Bytes of device scratch fsw_down uses for this shape: fp32 split-K partials in the small-M regime (required:
+ * FSW_E_WORKSPACE without them), a panel-blocked copy of H in the large-tile regime (optional: without it the kernel
+ * for row-major H runs, about 10 % slower), 0 otherwise. No counterpart in the reference, which has no down
+ * projection. */
 FSW_API size_t fsw_down_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF);
 
 /*

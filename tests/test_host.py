@@ -123,7 +123,9 @@ def test_variant_choice_by_regime(capi):
     # the down product with few output tiles and a deep K asks for split-K scratch; large or tiny M does not
     ws = capi.lib().fsw_down_workspace_bytes
     assert ws(0, 256, 4096, 14336) == 8 * 256 * 4096 * 4
-    assert ws(0, 8192, 4096, 14336) == 0 and ws(0, 16, 4096, 14336) == 0
+    # large-tile regime: scratch for a blocked copy of H (optional: without it fsw_down runs on row-major H)
+    assert ws(0, 8192, 4096, 14336) == L.fsw_blocked_bytes(8192, 14336) == 8192 * 14336 * 2
+    assert ws(0, 3000, 4096, 14336) == L.fsw_blocked_bytes(3000, 14336) and ws(0, 16, 4096, 14336) == 0
     assert capi.lib().fsw_mlp_workspace_bytes(0, 256, 4096, 14336) == 256 * 14336 * 2 + ws(0, 256, 4096, 14336)
 
 
