@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # L2<->fabric bytes per launch of the dominant kernel, from separate `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
 # runs scaled by a 1 GiB copy kernel (profiles/tiled_prefill_C3_hbm_traffic_pmc.md, skinny_decode_C4_kernel_trace.md);
 # not measurable in-process. C3: the gate/up kernel; C4: both decode kernels together.
-MEASURED_TRAFFIC_BYTES = {"C3": 3016230 * 1024 + 229376 * 1024, "C4": (230454 + 118324 + 448 + 128) * 1024}
+MEASURED_TRAFFIC_BYTES = {"C3": 2753094 * 1024 + 229376 * 1024, "C4": (230454 + 118324 + 448 + 128) * 1024}
 
 
 def parse():
