@@ -126,6 +126,7 @@ const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, i
   if (family < 0 || family > 1) return "invalid";
   const int v = resolve_variant(family, M, N_or_D);
   if (v == VARIANT_SKINNY) return decode_stream_wanted(family, M, N_or_D, K_or_FF) ? "decode_stream" : "skinny";
+  if ((v == 8 || v == 5) && g_forced_variant[family] < 0 && fsw::pair_ring_mode() == 2) return "pair16_256x256";
   return fsw::tiled_variant(v).name;
 }
 
@@ -194,6 +195,10 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
       if (fsw::decode_mlp_supported(da, 1)) return finish(fsw::launch_decode_mlp(dtype, da, (hipStream_t)stream, 1));
     }
     return finish(fsw::launch_skinny(dtype, true, a, nullptr, (hipStream_t)stream));
+  }
+  if (v == 8 && g_forced_variant[0] < 0 && fsw::pair_ring_mode() == 2) {
+    a.layout = 0;  // 256 x 256 tiles on row-major operands: the 16x16x32 pair ring with row-major activations
+    return finish(fsw::launch_tiled_blocked(dtype, true, a, (hipStream_t)stream));
   }
   return finish(fsw::launch_tiled(v, dtype, true, a, (hipStream_t)stream));
 }
@@ -265,6 +270,10 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
     a.splits = plan.splits;
     a.partial = (float*)workspace;
     return finish(fsw::launch_tiled_splitk(dtype, plan.tile, a, (hipStream_t)stream));
+  }
+  if (v == 5 && g_forced_variant[1] < 0 && fsw::pair_ring_mode() == 2) {
+    a.layout = 0;
+    return finish(fsw::launch_tiled_blocked(dtype, false, a, (hipStream_t)stream));
   }
   return finish(fsw::launch_tiled(v, dtype, false, a, (hipStream_t)stream));
 }

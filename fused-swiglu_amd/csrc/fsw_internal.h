@@ -42,6 +42,7 @@ const TiledVariant& tiled_variant(int variant);
 hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
 // gated: X blocked in (bit 0), H blocked out (bit 1) or row-major, W13 blocked (bit 2) or row-major: layouts 1, 3, 5, 7;
 // plain: H blocked in, W2 row-major (1) or blocked (5)
+int pair_ring_mode();  // kernel family behind the 256 x 256 tiles: 2 = 16x16x32 pair ring, 1 / 0 = 32x32x16 kernels
 hipError_t launch_tiled_blocked(int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
 // row-major [rows, k] (row stride ld elements) -> blocked; gated_order: W13's up/gate rows de-interleaved per panel
 hipError_t launch_block_rows(const void* src, long long ld, int rows, int k, void* dst, bool gated_order,

@@ -801,7 +801,9 @@ tiled_ring_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const 
 // PBLK: the weight operand is panel-blocked as well (prepacked; for the gated kernel in de-interleaved row order). It
 // then arrives like the activations, one 16 KB block per K tile, and keeps a ring of four 64-byte-row stages instead
 // of the pair slots (128 KB of LDS).
-template <class E, bool GATED, bool KTAIL, bool OBLK, bool PBLK = false>
+// QROW: the activation operand is row-major (callers without scratch for a blocked copy; few ragged activation
+// panels, where re-blocking does not pay): 64-byte requests per row and K tile, rows past nq read as zero.
+template <class E, bool GATED, bool KTAIL, bool OBLK, bool PBLK = false, bool QROW = false>
 __global__ void __launch_bounds__(256)
 tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
   constexpr int WP = 2, WQ = 2;
@@ -861,11 +863,17 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   const int pcq = t & 3;
   const int rbq = t >> 2;
   const int lcq = pcq ^ ((rbq >> 2) & 3);
-  const unsigned char* qbase = (const unsigned char*)a.Q + (long long)tq * nkt * QSTAGE;
-  const __amdgpu_buffer_rsrc_t qrs = make_rsrc(qbase, (long long)nkt * QSTAGE);
+  static_assert(!(QROW && (PBLK || OBLK)), "row-major activations: row-major weights and output only");
+  const unsigned char* qbase = QROW ? (const unsigned char*)a.Q + (long long)q0 * a.ldq * 2
+                                    : (const unsigned char*)a.Q + (long long)tq * nkt * QSTAGE;
+  const __amdgpu_buffer_rsrc_t qrs =
+      make_rsrc(qbase, QROW ? ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2 : (long long)nkt * QSTAGE);
   unsigned qoff[LQ];
 #pragma unroll
-  for (int j = 0; j < LQ; ++j) qoff[j] = (unsigned)(rbq + j * 64) * 64u + (unsigned)lcq * 16u;
+  for (int j = 0; j < LQ; ++j)
+    qoff[j] = QROW ? (unsigned)(rbq + j * 64) * (unsigned)a.ldq * 2u + (unsigned)lcq * 16u
+                   : (unsigned)(rbq + j * 64) * 64u + (unsigned)lcq * 16u;
+  constexpr int QSTEP = QROW ? 64 : QSTAGE;  // bytes between consecutive K tiles of the activation operand
 
   // operand fragment of a 16-row block: lane -> row r16, 16-byte K chunk c4 of the 32-element K tile
   const unsigned rd_p = PBLK ? (unsigned)((GATED ? wp * 64 : wp * 128) + r16) * 64u +
@@ -904,8 +912,9 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
         __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + (half * LPH + i) * 32 * 128 + wave * 1024), 16,
                                                  (int)(in ? poff[half * LPH + i] : OOB_OFFSET), pair * 128, 0, 0);
       } else {
+        const bool qin = !(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(qstage + (i - LPH) * 64 * 64 + wave * 1024), 16,
-                                                 (int)qoff[i - LPH], qt * QSTAGE, 0, 0);
+                                                 (int)(qin ? qoff[i - LPH] : OOB_OFFSET), qt * QSTEP, 0, 0);
       }
     }
   };
@@ -928,10 +937,11 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   };
   auto dma_q = [&](int qt_, unsigned char* qstage) {
     const int qt = qt_ < nkt ? qt_ : nkt - 1;
+    const bool qin = !(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k;
 #pragma unroll
     for (int j = 0; j < LQ; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(qstage + j * 64 * 64 + wave * 1024), 16, (int)qoff[j],
-                                               qt * QSTAGE, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(qstage + j * 64 * 64 + wave * 1024), 16,
+                                               (int)(qin ? qoff[j] : OOB_OFFSET), qt * QSTEP, 0, 0);
   };
 
   // two register sets of the 16 fragments of a K tile: [0..7] weight blocks, [8..15] activation blocks
@@ -1527,6 +1537,23 @@ hipError_t launch_pair16(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// both operands row-major
+template <class E, bool GATED>
+hipError_t launch_pair16_rowmajor(const GemmArgs& a, hipStream_t stream) {
+  const int tiles_p = (a.np + 255) / 256;
+  const int tiles_q = (a.nq + 255) / 256;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
+  if (a.k % 64 == 0) {
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, false, false, true>), grid, block, 0, stream, a, tiles_p,
+                       tiles_q, raster_group(GATED));
+  } else {
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, false, false, true>), grid, block, 0, stream, a, tiles_p,
+                       tiles_q, raster_group(GATED));
+  }
+  return hipGetLastError();
+}
+
 // both operands blocked (prepacked weights): the 16x16x32 kernel with a stage ring for the weights
 template <class E, bool GATED, bool OBLK>
 hipError_t launch_pair16_blocked(const GemmArgs& a, hipStream_t stream) {
@@ -1547,7 +1574,9 @@ hipError_t launch_blocked_typed(bool gated, const GemmArgs& a, hipStream_t strea
     if (gated && a.layout == 5) return launch_pair16_blocked<E, true, false>(a, stream);
     if (gated && a.layout == 7) return launch_pair16_blocked<E, true, true>(a, stream);
     if (!gated && a.layout == 5) return launch_pair16_blocked<E, false, false>(a, stream);
+    if (a.layout == 0) return gated ? launch_pair16_rowmajor<E, true>(a, stream) : launch_pair16_rowmajor<E, false>(a, stream);
   }
+  if (a.layout == 0) return hipErrorInvalidValue;
   if (g_pair_ring) {
     if (gated && a.layout == 1) return launch_pair<E, true, false>(a, stream);
     if (gated && a.layout == 3) return launch_pair<E, true, true>(a, stream);
@@ -1658,6 +1687,7 @@ hipError_t launch_block_rows(const void* src, long long ld, int rows, int k, voi
 
 void set_raster_group(int g) { g_raster_group = g > 0 ? g : 0; }
 void set_pair_ring(int mode) { g_pair_ring = mode < 0 || mode > 2 ? 2 : mode; }
+int pair_ring_mode() { return g_pair_ring; }
 int tiled_variant_count() { return (int)(sizeof(kVariants) / sizeof(kVariants[0])); }
 const TiledVariant& tiled_variant(int variant) { return kVariants[variant]; }
 

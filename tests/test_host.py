@@ -101,8 +101,8 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu(capi):
 
 def test_variant_choice_by_regime(capi):
     name = lambda fam, M, n, k: capi.variant_name(fam, 0, M, n, k)
-    assert name(0, 8192, 28672, 4096) == "ring_256x256"
-    assert name(1, 8192, 4096, 14336) == "dma_256x256"
+    assert name(0, 8192, 28672, 4096) == "pair16_256x256"
+    assert name(1, 8192, 4096, 14336) == "pair16_256x256"
     assert "256x256" in name(0, 4096, 22016, 4096)
     assert name(0, 512, 5632, 1024) == "dma_128x128"     # small problem: more, smaller tiles
     assert name(0, 16, 28672, 4096) == "skinny" and name(1, 1, 4096, 14336) == "skinny"
