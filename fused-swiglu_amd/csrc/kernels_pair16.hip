@@ -1,0 +1,407 @@
+// The prefill kernel of the dispatcher: 256 x 256 tiles on v_mfma_f32_16x16x32, weights in a ring of K-pair slots (or
+// 64-byte-row stages when prepacked), activations in a ring of four stages. Own translation unit: it is the largest
+// set of instances of the library and compiles beside kernels_tiled.hip, which keeps the 32x32x16 kernels.
+#include <type_traits>
+
+#include "fsw_internal.h"
+#include "fsw_device.h"
+
+namespace fsw {
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+// ---- pair ring on v_mfma_f32_16x16x32 ----------------------------------------------------------------------------
+// Same tile, copy engine, LDS layouts and rings as tiled_pair_kernel below; the wave tile of 128 x 128 is 8 x 8
+// blocks of 16 x 16 and ONE MFMA covers the whole 32-deep K tile. Per FLOP the 16x16x32 instruction moves half the
+// accumulator registers of 32x32x16 (and twice the operand registers: 20 % less register-file traffic in total), and
+// under the board's power cap that is what sets the clock: a register-only loop of either instruction issues at the
+// same rate with all-zero operands (2445 vs 2480 TFLOP/s) and sustains 2090 vs 1822 TFLOP/s with random operands.
+// Accumulators are a two-dimensional array indexed by constants only (a flat array made the register allocator move
+// accumulators between MFMAs).
+// [the description of the rings follows at tiled_pair_kernel]
+// PBLK: the weight operand is panel-blocked as well (prepacked; for the gated kernel in de-interleaved row order). It
+// then arrives like the activations, one 16 KB block per K tile, and keeps a ring of four 64-byte-row stages instead
+// of the pair slots (128 KB of LDS).
+// QROW: the activation operand is row-major (callers without scratch for a blocked copy; few ragged activation
+// panels, where re-blocking does not pay): 64-byte requests per row and K tile, rows past nq read as zero.
+template <class E, bool GATED, bool KTAIL, bool OBLK, bool PBLK = false, bool QROW = false>
+__global__ void __launch_bounds__(256)
+tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
+  constexpr int WP = 2, WQ = 2;
+  constexpr int NB = 8;  // 16-row blocks per wave and operand
+  constexpr int BP = 256, BQ = 256;
+  constexpr int PSLOT = BP * 128, QSTAGE = BQ * 64;
+  constexpr int LPH = 4;  // weight copy instructions per wave per HALF pair (8 rows x 128 B each)
+  constexpr int LQ = 4;   // activation copy instructions per wave per K tile (16 rows x 64 B each)
+  constexpr int NL = LPH + LQ;
+  static_assert(!OBLK || GATED, "only H is ever written blocked");
+  static_assert(!PBLK || !KTAIL, "blocked operands are zero padded in K");
+  constexpr int PSTAGE = BP * 64;
+  constexpr int PBUF = PBLK ? PSTAGE : PSLOT;
+
+  __shared__ __align__(1024) unsigned char ps0[PBUF];
+  __shared__ __align__(1024) unsigned char ps1[PBUF];
+  __shared__ __align__(1024) unsigned char ps2[PBUF];
+  __shared__ alignas(PBLK ? 1024 : 16) unsigned char ps3[PBLK ? PSTAGE : 16];
+  __shared__ __align__(1024) unsigned char qs0[QSTAGE];
+  __shared__ __align__(1024) unsigned char qs1[QSTAGE];
+  __shared__ __align__(1024) unsigned char qs2[QSTAGE];
+  __shared__ __align__(1024) unsigned char qs3[QSTAGE];
+  unsigned char* const ps[4] = {ps0, ps1, ps2, ps3};
+  unsigned char* const qs[4] = {qs0, qs1, qs2, qs3};
+
+  const int t = threadIdx.x;
+  const int lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wq = wave % WQ;
+  const int wp = wave / WQ;
+  const int r16 = lane & 15;
+  const int c4 = lane >> 4;
+
+  int tp, tq;
+  tile_coords(blockIdx.x, tiles_p, tiles_q, group, tp, tq);
+  const int p0 = tp * BP;
+  const int q0 = tq * BQ;
+  const int nkt = (a.k + 31) / 32;
+  const int npair = (nkt + 1) / 2;
+
+  // weight copy: lane -> chunk position pcp of row rbp (+ 32 j), fetches logical chunk lcp of the 128-byte line
+  const int pcp = t & 7;
+  const int rbp = t >> 3;
+  const int lcp = pcp ^ ((rbp >> 1) & 7);
+  const unsigned char* pbase = PBLK ? (const unsigned char*)a.P + (long long)tp * nkt * PSTAGE
+                                    : (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
+  const __amdgpu_buffer_rsrc_t prs =
+      make_rsrc(pbase, PBLK ? (long long)nkt * PSTAGE : ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
+  unsigned poff[2 * LPH];
+#pragma unroll
+  for (int j = 0; j < 2 * LPH; ++j) {
+    const int r = rbp + j * 32;
+    const int grow = GATED ? (r < BP / 2 ? 2 * r : 2 * (r - BP / 2) + 1) : r;
+    poff[j] = (unsigned)grow * (unsigned)a.ldp * 2u + (unsigned)lcp * 16u;
+  }
+  // activation copy from the blocked panel: lane -> chunk position pcq of row rbq (+ 64 j)
+  const int pcq = t & 3;
+  const int rbq = t >> 2;
+  const int lcq = pcq ^ ((rbq >> 2) & 3);
+  static_assert(!(QROW && (PBLK || OBLK)), "row-major activations: row-major weights and output only");
+  const unsigned char* qbase = QROW ? (const unsigned char*)a.Q + (long long)q0 * a.ldq * 2
+                                    : (const unsigned char*)a.Q + (long long)tq * nkt * QSTAGE;
+  const __amdgpu_buffer_rsrc_t qrs =
+      make_rsrc(qbase, QROW ? ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2 : (long long)nkt * QSTAGE);
+  unsigned qoff[LQ];
+#pragma unroll
+  for (int j = 0; j < LQ; ++j)
+    qoff[j] = QROW ? (unsigned)(rbq + j * 64) * (unsigned)a.ldq * 2u + (unsigned)lcq * 16u
+                   : (unsigned)(rbq + j * 64) * 64u + (unsigned)lcq * 16u;
+  constexpr int QSTEP = QROW ? 64 : QSTAGE;  // bytes between consecutive K tiles of the activation operand
+
+  // operand fragment of a 16-row block: lane -> row r16, 16-byte K chunk c4 of the 32-element K tile
+  const unsigned rd_p = PBLK ? (unsigned)((GATED ? wp * 64 : wp * 128) + r16) * 64u +
+                                   (unsigned)((c4 ^ ((r16 >> 2) & 3)) * 16)
+                             : (unsigned)((GATED ? wp * 64 : wp * 128) + r16) * 128u;
+  const unsigned rd_q = (unsigned)(wq * 128 + r16) * 64u + (unsigned)((c4 ^ ((r16 >> 2) & 3)) * 16);
+  unsigned xp[2];  // [half of the pair]
+#pragma unroll
+  for (int h = 0; h < 2; ++h) xp[h] = (unsigned)((((h << 2) | c4) ^ ((r16 >> 1) & 7)) * 16);
+  auto p_block_off = [](int f) -> unsigned {
+    constexpr unsigned RB = PBLK ? 64 : 128;  // bytes per weight row in LDS
+    if (GATED) return (unsigned)(f < NB / 2 ? f * 16 : BP / 2 + (f - NB / 2) * 16) * RB;
+    return (unsigned)(f * 16) * RB;
+  };
+
+  f32x4 acc[NB][NB];
+#pragma unroll
+  for (int f = 0; f < NB; ++f)
+#pragma unroll
+    for (int g = 0; g < NB; ++g) acc[f][g] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // copy instruction idx of iteration kt: 0..3 = half (kt & 1) of weight pair (kt >> 1) + 2, 4..7 = activation tile
+  // kt + 3. Past the end both re-read the last pair / tile (never consumed).
+  auto dma = [&](int kt, unsigned char* pslot, unsigned char* qstage, auto lo_c, auto hi_c) {
+    constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
+    const int pair = (kt >> 1) + 2 < npair ? (kt >> 1) + 2 : npair - 1;
+    const int half = kt & 1;
+    const int qt = kt + 3 < nkt ? kt + 3 : nkt - 1;
+    const bool in = !KTAIL || (pair * 64 + lcp * 8) < a.k;
+#pragma unroll
+    for (int i = LO; i < HI; ++i) {
+      if (i < LPH && PBLK) {  // weight tile kt + 3, copied like an activation tile
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + i * 64 * 64 + wave * 1024), 16, (int)qoff[i],
+                                                 qt * PSTAGE, 0, 0);
+      } else if (i < LPH) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + (half * LPH + i) * 32 * 128 + wave * 1024), 16,
+                                                 (int)(in ? poff[half * LPH + i] : OOB_OFFSET), pair * 128, 0, 0);
+      } else {
+        const bool qin = !(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(qstage + (i - LPH) * 64 * 64 + wave * 1024), 16,
+                                                 (int)(qin ? qoff[i - LPH] : OOB_OFFSET), qt * QSTEP, 0, 0);
+      }
+    }
+  };
+  // prologue copies: a whole weight pair / one activation tile
+  auto dma_pair = [&](int pair_, unsigned char* pslot, int j_lo, int j_hi) {
+    const int pair = pair_ < npair ? pair_ : npair - 1;
+    const bool in = !KTAIL || (pair * 64 + lcp * 8) < a.k;
+#pragma unroll
+    for (int j = 0; j < 2 * LPH; ++j)
+      if (j >= j_lo && j < j_hi)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + j * 32 * 128 + wave * 1024), 16,
+                                                 (int)(in ? poff[j] : OOB_OFFSET), pair * 128, 0, 0);
+  };
+  auto dma_pb = [&](int pt_, unsigned char* pstage) {
+    const int pt = pt_ < nkt ? pt_ : nkt - 1;
+#pragma unroll
+    for (int j = 0; j < LPH; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pstage + j * 64 * 64 + wave * 1024), 16, (int)qoff[j],
+                                               pt * PSTAGE, 0, 0);
+  };
+  auto dma_q = [&](int qt_, unsigned char* qstage) {
+    const int qt = qt_ < nkt ? qt_ : nkt - 1;
+    const bool qin = !(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k;
+#pragma unroll
+    for (int j = 0; j < LQ; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(qstage + j * 64 * 64 + wave * 1024), 16,
+                                               (int)(qin ? qoff[j] : OOB_OFFSET), qt * QSTEP, 0, 0);
+  };
+
+  // two register sets of the 16 fragments of a K tile: [0..7] weight blocks, [8..15] activation blocks
+  u32x4 fr[2][2 * NB];
+  using C0 = std::integral_constant<int, 0>;
+  using CH = std::integral_constant<int, LPH>;
+  // The barrier sits in the middle of the iteration. At the barrier of iteration kt everything issued up to
+  // iteration kt - 2 has landed (tile kt + 1 and its weight pair among it); the copies of iteration kt - 1 and of
+  // this one stay in flight. lgkmcnt(0): this wave's reads of tile kt (issued in the second half of
+  // iteration kt - 1) are complete, so its stage may be refilled from the next iteration on.
+  constexpr int VM = NL + NL;
+  constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
+
+  // Fragment read by index: weight block 0, the 8 activation blocks, then weight blocks 1 .. 7: the order the MFMAs
+  // (f major, g minor) first need them.
+  auto read_one = [&](int set, int idx, const unsigned char* pslot, int half, const unsigned char* qstage) {
+    if (idx == 0) {
+      fr[set][0] = *(const u32x4*)(pslot + rd_p + p_block_off(0) + (PBLK ? 0u : xp[half]));
+    } else if (idx <= NB) {
+      fr[set][NB + idx - 1] = *(const u32x4*)(qstage + rd_q + (idx - 1) * 16 * 64);
+    } else {
+      fr[set][idx - NB] = *(const u32x4*)(pslot + rd_p + p_block_off(idx - NB) + (PBLK ? 0u : xp[half]));
+    }
+  };
+  auto mma_one = [&](int set, int i) {
+    E::mfma16_acc(acc[i / NB][i % NB], fr[set][i / NB], fr[set][NB + i % NB]);
+  };
+  // iteration j (mod 12) of the unrolled loop, K tile kt = base + j, fragments of tile kt in register set j & 1.
+  // First half: the 32 MFMAs of weight blocks 0 .. 3 with the eight copies between them (one per four MFMAs);
+  // barrier; second half: the 32 MFMAs of weight blocks 4 .. 7 with the 16 fragment reads of tile kt + 1 (one per two
+  // MFMAs). The scheduler is fenced after every group, so this is the issue order. (A copy next to a read between two
+  // 16-cycle MFMAs — s_mov m0, the copy, the read, a wait — does not fit their shadow.)
+  auto iteration = [&](auto j_c, int kt) {
+    constexpr int J = decltype(j_c)::value;
+    constexpr int SET = J & 1;
+    unsigned char* const p_nxt = PBLK ? ps[(J + 1) & 3] : ps[((J + 1) >> 1) % 3];
+    unsigned char* const p_fill = PBLK ? ps[(J + 3) & 3] : ps[((J >> 1) + 2) % 3];
+    unsigned char* const q_nxt = qs[(J + 1) & 3];
+    unsigned char* const q_fill = qs[(J + 3) & 3];
+#define FSW_P16_GROUP(G)                                                                                      \
+    mma_one(SET, 8 * (G) + 0);                                                                                 \
+    mma_one(SET, 8 * (G) + 1);                                                                                 \
+    dma(kt, p_fill, q_fill, std::integral_constant<int, 2 * (G)>{}, std::integral_constant<int, 2 * (G) + 1>{}); \
+    __builtin_amdgcn_sched_barrier(0);                                                                         \
+    mma_one(SET, 8 * (G) + 2);                                                                                 \
+    mma_one(SET, 8 * (G) + 3);                                                                                 \
+    mma_one(SET, 8 * (G) + 4);                                                                                 \
+    mma_one(SET, 8 * (G) + 5);                                                                                 \
+    dma(kt, p_fill, q_fill, std::integral_constant<int, 2 * (G) + 1>{}, std::integral_constant<int, 2 * (G) + 2>{}); \
+    __builtin_amdgcn_sched_barrier(0);                                                                         \
+    mma_one(SET, 8 * (G) + 6);                                                                                 \
+    mma_one(SET, 8 * (G) + 7);                                                                                 \
+    __builtin_amdgcn_sched_barrier(0);
+    FSW_P16_GROUP(0)
+    FSW_P16_GROUP(1)
+    FSW_P16_GROUP(2)
+    FSW_P16_GROUP(3)
+#undef FSW_P16_GROUP
+    asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(WAIT_IMM) : "memory");
+#pragma unroll
+    for (int r = 0; r < 2 * NB; ++r) {
+      mma_one(SET, 4 * NB + 2 * r);
+      read_one(SET ^ 1, r, p_nxt, (J + 1) & 1, q_nxt);
+      mma_one(SET, 4 * NB + 2 * r + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  if (nkt > 0) {
+    // fill in the order the loop would have issued it: [pair 0, tile 0] [pair 1 first half, tile 1] [pair 1 second
+    // half, tile 2]; then pair 0 and tile 0 have landed when 16 copies are still in flight
+    if constexpr (PBLK) {
+      dma_pb(0, ps0);
+      dma_q(0, qs0);
+      dma_pb(1, ps1);
+      dma_q(1, qs1);
+      dma_pb(2, ps2);
+      dma_q(2, qs2);
+    } else {
+      dma_pair(0, ps0, 0, 2 * LPH);
+      dma_q(0, qs0);
+      dma_pair(1, ps1, 0, LPH);
+      dma_q(1, qs1);
+      dma_pair(1, ps1, LPH, 2 * LPH);
+      dma_q(2, qs2);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NL) : "memory");
+#pragma unroll
+    for (int i = 0; i < 2 * NB; ++i) read_one(0, i, ps0, 0, qs0);
+  }
+  int kt = 0;
+  for (; kt + 11 < nkt; kt += 12) {
+    iteration(std::integral_constant<int, 0>{}, kt);
+    iteration(std::integral_constant<int, 1>{}, kt + 1);
+    iteration(std::integral_constant<int, 2>{}, kt + 2);
+    iteration(std::integral_constant<int, 3>{}, kt + 3);
+    iteration(std::integral_constant<int, 4>{}, kt + 4);
+    iteration(std::integral_constant<int, 5>{}, kt + 5);
+    iteration(std::integral_constant<int, 6>{}, kt + 6);
+    iteration(std::integral_constant<int, 7>{}, kt + 7);
+    iteration(std::integral_constant<int, 8>{}, kt + 8);
+    iteration(std::integral_constant<int, 9>{}, kt + 9);
+    iteration(std::integral_constant<int, 10>{}, kt + 10);
+    iteration(std::integral_constant<int, 11>{}, kt + 11);
+  }
+#define FSW_PAIR16_TAIL(J)                                     \
+  if (kt < nkt) {                                            \
+    iteration(std::integral_constant<int, J>{}, kt);         \
+    ++kt;                                                    \
+  }
+  FSW_PAIR16_TAIL(0)
+  FSW_PAIR16_TAIL(1)
+  FSW_PAIR16_TAIL(2)
+  FSW_PAIR16_TAIL(3)
+  FSW_PAIR16_TAIL(4)
+  FSW_PAIR16_TAIL(5)
+  FSW_PAIR16_TAIL(6)
+  FSW_PAIR16_TAIL(7)
+  FSW_PAIR16_TAIL(8)
+  FSW_PAIR16_TAIL(9)
+  FSW_PAIR16_TAIL(10)
+#undef FSW_PAIR16_TAIL
+
+  // epilogue: a lane owns activation row r16 of each block column and 4 consecutive features (4 c4 ..) per block row
+  mfma_drain();
+  if constexpr (OBLK) {
+    // H panel-blocked (see store_tile_blocked): every row of the panel and every feature up to the next multiple
+    // of 32 is written; padding comes out of zero operand rows
+    const int nblocks = (a.np / 2 + 31) >> 5;
+    unsigned char* O = (unsigned char*)a.O;
+#pragma unroll
+    for (int g = 0; g < NB; ++g) {
+      const int row = wq * 128 + g * 16 + r16;
+#pragma unroll
+      for (int f = 0; f < NB / 2; ++f) {
+        const int blk = tp * 4 + wp * 2 + (f >> 1);
+        if (blk < nblocks) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = acc[f][g][e] * silu_f32(acc[f + NB / 2][g][e]);
+          u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
+          *(u32x2*)(O + (((long long)tq * nblocks + blk) * 256 + row) * 64 + (f & 1) * 32 + c4 * 8) = pk;
+        }
+      }
+    }
+  } else {
+    unsigned short* O = (unsigned short*)a.O;
+    constexpr int FO = GATED ? NB / 2 : NB;
+    const int nout = GATED ? a.np / 2 : a.np;
+    const bool vec_ok = ((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 7) == 0);
+#pragma unroll
+    for (int g = 0; g < NB; ++g) {
+      const int m = q0 + wq * 128 + g * 16 + r16;
+      if (m >= a.nq) continue;
+      unsigned short* orow = O + (long long)m * a.ldo;
+#pragma unroll
+      for (int f = 0; f < FO; ++f) {
+        const int n = (GATED ? p0 / 2 + wp * 64 : p0 + wp * 128) + f * 16 + c4 * 4;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = GATED ? acc[f][g][e] * silu_f32(acc[f + FO][g][e]) : acc[f][g][e];
+        if (vec_ok && n + 3 < nout) {
+          u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
+          *(u32x2*)(orow + n) = pk;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < nout) orow[n + e] = E::cvt1(v[e]);
+        }
+      }
+    }
+  }
+}
+
+
+namespace {
+
+template <class E, bool GATED, bool OBLK>
+hipError_t launch_pair16_rowmajor_w(const GemmArgs& a, hipStream_t stream) {
+  const int tiles_p = (a.np + 255) / 256;
+  const int tiles_q = (a.nq + 255) / 256;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
+  if (a.k % 64 == 0) {
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK>), grid, block, 0, stream, a, tiles_p, tiles_q,
+                       raster_group(GATED));
+  } else {
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, OBLK>), grid, block, 0, stream, a, tiles_p, tiles_q,
+                       raster_group(GATED));
+  }
+  return hipGetLastError();
+}
+
+// both operands row-major
+template <class E, bool GATED>
+hipError_t launch_pair16_rowmajor(const GemmArgs& a, hipStream_t stream) {
+  const int tiles_p = (a.np + 255) / 256;
+  const int tiles_q = (a.nq + 255) / 256;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
+  if (a.k % 64 == 0) {
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, false, false, true>), grid, block, 0, stream, a, tiles_p,
+                       tiles_q, raster_group(GATED));
+  } else {
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, false, false, true>), grid, block, 0, stream, a, tiles_p,
+                       tiles_q, raster_group(GATED));
+  }
+  return hipGetLastError();
+}
+
+// both operands blocked (prepacked weights): the 16x16x32 kernel with a stage ring for the weights
+template <class E, bool GATED, bool OBLK>
+hipError_t launch_pair16_blocked(const GemmArgs& a, hipStream_t stream) {
+  const int tiles_p = (a.np + 255) / 256;
+  const int tiles_q = (a.nq + 255) / 256;
+  if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
+  hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK, true>), dim3((unsigned)(tiles_p * tiles_q)), dim3(256), 0,
+                     stream, a, tiles_p, tiles_q, raster_group(GATED));
+  return hipGetLastError();
+}
+
+template <class E>
+hipError_t launch_pair16_typed(bool gated, const GemmArgs& a, hipStream_t stream) {
+  if (gated && a.layout == 1) return launch_pair16_rowmajor_w<E, true, false>(a, stream);
+  if (gated && a.layout == 3) return launch_pair16_rowmajor_w<E, true, true>(a, stream);
+  if (!gated && a.layout == 1) return launch_pair16_rowmajor_w<E, false, false>(a, stream);
+  if (gated && a.layout == 5) return launch_pair16_blocked<E, true, false>(a, stream);
+  if (gated && a.layout == 7) return launch_pair16_blocked<E, true, true>(a, stream);
+  if (!gated && a.layout == 5) return launch_pair16_blocked<E, false, false>(a, stream);
+  if (a.layout == 0) return gated ? launch_pair16_rowmajor<E, true>(a, stream) : launch_pair16_rowmajor<E, false>(a, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+// GemmArgs::layout: bit 0 = activations blocked, bit 1 = output blocked (gated only), bit 2 = weights blocked
+hipError_t launch_pair16(int dtype, bool gated, const GemmArgs& a, hipStream_t stream) {
+  return dtype == 0 ? launch_pair16_typed<Bf16>(gated, a, stream) : launch_pair16_typed<Fp16>(gated, a, stream);
+}
+
+}  // namespace fsw
