@@ -11,14 +11,27 @@ namespace fsw {
 typedef __attribute__((address_space(3))) void lds_void;
 
 // ---- pair ring on v_mfma_f32_16x16x32 ----------------------------------------------------------------------------
-// Same tile, copy engine, LDS layouts and rings as tiled_pair_kernel below; the wave tile of 128 x 128 is 8 x 8
-// blocks of 16 x 16 and ONE MFMA covers the whole 32-deep K tile. Per FLOP the 16x16x32 instruction moves half the
-// accumulator registers of 32x32x16 (and twice the operand registers: 20 % less register-file traffic in total), and
-// under the board's power cap that is what sets the clock: a register-only loop of either instruction issues at the
-// same rate with all-zero operands (2445 vs 2480 TFLOP/s) and sustains 2090 vs 1822 TFLOP/s with random operands.
-// Accumulators are a two-dimensional array indexed by constants only (a flat array made the register allocator move
-// accumulators between MFMAs).
-// [the description of the rings follows at tiled_pair_kernel]
+// 256 x 256 workgroup tile, 4 waves of 128 x 128, K tiles of 32 elements. The wave tile is 8 x 8 blocks of 16 x 16 and
+// ONE MFMA covers the whole 32-deep K tile. Per FLOP the 16x16x32 instruction moves half the accumulator registers of
+// 32x32x16 (and twice the operand registers: 20 % less register-file traffic in total), and under the board's power
+// cap that is what sets the clock: a register-only loop of either instruction issues at the same rate with all-zero
+// operands (2445 vs 2480 TFLOP/s) and sustains 2090 vs 1822 TFLOP/s with random operands. Accumulators are a
+// two-dimensional array indexed by constants only (a flat array made the register allocator move accumulators
+// between MFMAs), and the MFMA is written out with its destination tied to the addend (mfma16_acc).
+//
+// Operands go global -> LDS with buffer_load ... lds. The activation operand is panel-blocked (blocks of
+// [256 rows][32 elements], 16 KB contiguous) and keeps a ring of four 16 KB stages; a tile is issued three iterations
+// before it is multiplied. The weight operand is ROW-MAJOR: read 32 K elements at a time it would yield 64-byte
+// requests, half a cache line each, so it is fetched in K PAIRS (64 elements = one 128-byte line per row) into a ring
+// of three 32 KB pair slots, half a pair per iteration, four to three iterations ahead. The slot/stage pattern
+// repeats every 12 K tiles (lcm of 6 and 4): the loop is unrolled twelvefold with every LDS address a compile-time
+// constant. 160 KB of LDS.
+// LDS layouts: pair slot = [256 rows][128 B], chunk c of row r at position c ^ ((r >> 1) & 7); activation stage =
+// [256 rows][64 B], chunk c at c ^ ((r >> 2) & 3): the 16 rows a fragment read touches at one logical chunk cover
+// the 64 banks once. The swizzle is applied on the global side of the copy (which lane fetches which chunk), since
+// an LDS-DMA instruction writes lane i at base + 16 i. For the gated kernel the even ("up") weight rows of a tile go
+// to LDS rows 0..127 and the odd ("gate") rows to 128..255; a wave multiplies 64 of each against the same activation
+// fragments, so up and gate of one output land in the same lane and register index.
 // PBLK: the weight operand is panel-blocked as well (prepacked; for the gated kernel in de-interleaved row order). It
 // then arrives like the activations, one 16 KB block per K tile, and keeps a ring of four 64-byte-row stages instead
 // of the pair slots (128 KB of LDS).
@@ -338,11 +351,11 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
   }
 }
 
-
 namespace {
 
+// activations blocked, weights row-major
 template <class E, bool GATED, bool OBLK>
-hipError_t launch_pair16_rowmajor_w(const GemmArgs& a, hipStream_t stream) {
+hipError_t launch_pair16_blocked_x(const GemmArgs& a, hipStream_t stream) {
   const int tiles_p = (a.np + 255) / 256;
   const int tiles_q = (a.nq + 255) / 256;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
@@ -376,7 +389,7 @@ hipError_t launch_pair16_rowmajor(const GemmArgs& a, hipStream_t stream) {
 
 // both operands blocked (prepacked weights): the 16x16x32 kernel with a stage ring for the weights
 template <class E, bool GATED, bool OBLK>
-hipError_t launch_pair16_blocked(const GemmArgs& a, hipStream_t stream) {
+hipError_t launch_pair16_blocked_xw(const GemmArgs& a, hipStream_t stream) {
   const int tiles_p = (a.np + 255) / 256;
   const int tiles_q = (a.nq + 255) / 256;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
@@ -387,12 +400,12 @@ hipError_t launch_pair16_blocked(const GemmArgs& a, hipStream_t stream) {
 
 template <class E>
 hipError_t launch_pair16_typed(bool gated, const GemmArgs& a, hipStream_t stream) {
-  if (gated && a.layout == 1) return launch_pair16_rowmajor_w<E, true, false>(a, stream);
-  if (gated && a.layout == 3) return launch_pair16_rowmajor_w<E, true, true>(a, stream);
-  if (!gated && a.layout == 1) return launch_pair16_rowmajor_w<E, false, false>(a, stream);
-  if (gated && a.layout == 5) return launch_pair16_blocked<E, true, false>(a, stream);
-  if (gated && a.layout == 7) return launch_pair16_blocked<E, true, true>(a, stream);
-  if (!gated && a.layout == 5) return launch_pair16_blocked<E, false, false>(a, stream);
+  if (gated && a.layout == 1) return launch_pair16_blocked_x<E, true, false>(a, stream);
+  if (gated && a.layout == 3) return launch_pair16_blocked_x<E, true, true>(a, stream);
+  if (!gated && a.layout == 1) return launch_pair16_blocked_x<E, false, false>(a, stream);
+  if (gated && a.layout == 5) return launch_pair16_blocked_xw<E, true, false>(a, stream);
+  if (gated && a.layout == 7) return launch_pair16_blocked_xw<E, true, true>(a, stream);
+  if (!gated && a.layout == 5) return launch_pair16_blocked_xw<E, false, false>(a, stream);
   if (a.layout == 0) return gated ? launch_pair16_rowmajor<E, true>(a, stream) : launch_pair16_rowmajor<E, false>(a, stream);
   return hipErrorInvalidValue;
 }
