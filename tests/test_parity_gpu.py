@@ -547,3 +547,31 @@ def test_forward_replays_from_a_hip_graph(capi, shape):
         torch.cuda.synchronize()
         assert torch.equal(Y, eager), "replay %d differs from the eager forward" % rep
     oracle.assert_parity(Y, oracle.ref_mlp(X.cpu(), inp["W13"], inp["W2"], torch.float64), "graph replay")
+
+
+def test_large_tiles_on_row_major_activations(capi):
+    """256 x 256 tiles with ROW-MAJOR activations: fsw_gateup for a ragged M below 1024 (no re-blocking there) and
+    fsw_down without the optional scratch for a blocked copy of H. Both against the oracle, and the down projection
+    bit for bit against the call that does get the scratch."""
+    L = capi.lib()
+    M, d, ff = 600, 520, 12800           # 3 x 100 tiles of 256 x 256, K = 520 is not a multiple of 64
+    assert capi.variant_name(0, 0, M, 2 * ff, d) == "pair16_256x256" and L.fsw_gateup_workspace_bytes(0, M, 2 * ff, d) == 0
+    inp = fsw_weights.make_inputs(M, d, ff, torch.bfloat16, seed=31, x_scale=0.5)
+    g = to_dev(inp)
+    H = capi.gateup(g["X"], g["W13"])
+    rows = torch.arange(0, M, 7)
+    C = inp["X"][rows].double() @ inp["W13"].double().T
+    assert_one_rounding(H[rows.to(DEV)], C[:, 0::2] * torch.nn.functional.silu(C[:, 1::2]), torch.bfloat16, "row-major X, 256x256")
+    M2, D2, FF2 = 3300, 4096, 264         # 16 x 13 tiles, ragged M, K = 264
+    assert capi.variant_name(1, 0, M2, D2, FF2) == "pair16_256x256"
+    gen = torch.Generator().manual_seed(32)
+    Hh = (torch.randn(M2, FF2, generator=gen) * 0.5).to(torch.float16)
+    W2 = (torch.randn(D2, FF2, generator=gen) / FF2 ** 0.5).to(torch.float16)
+    Hd, W2d = Hh.to(DEV), W2.to(DEV)
+    Y0 = torch.empty(M2, D2, dtype=torch.float16, device=DEV)
+    s = torch.cuda.current_stream().cuda_stream
+    capi.check(L.fsw_down(1, M2, D2, FF2, Hd.data_ptr(), FF2, W2d.data_ptr(), FF2, Y0.data_ptr(), D2, None, 0, s))
+    Y1 = capi.down(Hd, W2d)               # with scratch: H re-blocked first
+    assert torch.equal(Y0, Y1)
+    rows = torch.arange(0, M2, 31)
+    assert_one_rounding(Y0[rows.to(DEV)], Hh[rows].double() @ W2.double().T, torch.float16, "row-major H, 256x256")
