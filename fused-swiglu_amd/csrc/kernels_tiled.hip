@@ -359,7 +359,7 @@ tiled_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int g
 // tell reads of the live stage from DMA writes into the other one.
 typedef __attribute__((address_space(3))) void lds_void;
 
-template <class E, bool GATED, bool KTAIL, int WP, int WQ, int FP, int FQ, bool STREAM_W = false>
+template <class E, bool GATED, bool KTAIL, int WP, int WQ, int FP, int FQ, bool STREAM_W = false, int NS = 2>
 __global__ void __launch_bounds__(WP* WQ * 64)
 tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
   constexpr int NT = WP * WQ * 64;
@@ -373,10 +373,13 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
   constexpr int STAGE = (BP + BQ) * ROWB;
   static_assert(BP % RSTEP == 0 && BQ % RSTEP == 0 && RSTEP % 16 == 0, "copy mapping");
   static_assert(!GATED || (FP % 2 == 0), "gated kernel pairs fragments");
-  static_assert(2 * STAGE <= 160 * 1024, "LDS budget of a gfx950 CU");
+  static_assert(NS >= 2 && NS <= 5 && NS * STAGE <= 160 * 1024, "LDS budget of a gfx950 CU");
 
   __shared__ __align__(1024) unsigned char lds0[STAGE];
   __shared__ __align__(1024) unsigned char lds1[STAGE];
+  __shared__ alignas(NS > 2 ? 1024 : 16) unsigned char lds2[NS > 2 ? STAGE : 16];
+  __shared__ alignas(NS > 3 ? 1024 : 16) unsigned char lds3[NS > 3 ? STAGE : 16];
+  __shared__ alignas(NS > 4 ? 1024 : 16) unsigned char lds4[NS > 4 ? STAGE : 16];
 
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -528,15 +531,79 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
     }
   };
 
-  if (nkt > 0) dma(lds0, 0);
-  __syncthreads();
-  if (nkt > 0) f_read(0, lds0, 0);
-  int kt = 0;
-  for (; kt + 1 < nkt; kt += 2) {
-    iteration(lds0, lds1, kt);
-    iteration(lds1, lds0, kt + 1);
+  // NS stages: two for the compute-bound uses; three when every weight byte comes from HBM exactly once (a single
+  // tile of activation rows, weights streamed non-temporally): the copy of tile kt + 2 is issued while tile kt is
+  // multiplied, which doubles the bytes in flight per workgroup. Measured at 4096 x 28672, gate/up: M = 65: 67.6 ->
+  // 43.9 us, M = 128: 67.0 -> 49.0 us (a fourth stage: level). The split-K down projection keeps two stages (three
+  // cost it an LDS-limited workgroup per CU: 36.7 -> 40.4 us).
+  if constexpr (NS == 2) {
+    if (nkt > 0) dma(lds0, 0);
+    __syncthreads();
+    if (nkt > 0) f_read(0, lds0, 0);
+    int kt = 0;
+    for (; kt + 1 < nkt; kt += 2) {
+      iteration(lds0, lds1, kt);
+      iteration(lds1, lds0, kt + 1);
+    }
+    if (kt < nkt) iteration(lds0, lds1, kt);
+  } else {
+    unsigned char* const ring[5] = {lds0, lds1, lds2, lds3, lds4};
+    constexpr int VM = (NS - 2) * NL;
+    static_assert(VM <= 63, "vmcnt is a 6-bit counter");
+    constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
+    auto ring_iteration = [&](unsigned char* cur, unsigned char* nxt, unsigned char* fill, int kt) {
+      dma(fill, kt + NS - 1);
+      f_read(1, cur, 1);
+      mma(0, 0, FP);
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, (NL + NR - 1) / NR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      f_read(0, cur, 2);
+      mma(1, 0, FP);
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      f_read(1, cur, 3);
+      mma(0, 0, FP);
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      mma(1, 0, HF);
+      asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(WAIT_IMM) : "memory");
+      f_read(0, nxt, 0);
+      mma(1, HF, FP);
+#pragma unroll
+      for (int i = 0; i < (FP - HF) * FQ; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, (NR + (FP - HF) * FQ - 1) / ((FP - HF) * FQ), 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+    };
+    if (nkt > 0) {
+#pragma unroll
+      for (int j = 0; j < NS - 1; ++j) dma(ring[j], j);
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NS - 2) * NL) : "memory");
+      f_read(0, lds0, 0);
+    }
+    int kt = 0;
+    for (; kt + NS - 1 < nkt; kt += NS) {
+#pragma unroll
+      for (int j = 0; j < NS; ++j) ring_iteration(ring[j], ring[(j + 1) % NS], ring[(j + NS - 1) % NS], kt + j);
+    }
+#pragma unroll
+    for (int j = 0; j < NS - 1; ++j) {
+      if (kt < nkt) {
+        ring_iteration(ring[j], ring[(j + 1) % NS], ring[(j + NS - 1) % NS], kt);
+        ++kt;
+      }
+    }
   }
-  if (kt < nkt) iteration(lds0, lds1, kt);
 
   if constexpr (!GATED) {
     if (a.splits > 1) {
@@ -1088,6 +1155,7 @@ const TiledVariant kVariants[] = {
     {"dma8w_256x256", 256, 256, 512},
     {"ring5_256x256", 256, 256, 256},  // five-stage ring: all 160 KB of LDS, four K tiles in flight
     {"ring5_256x192", 256, 192, 256},  // 192 activation rows: fewer padded rows / idle CUs for some M (see pick_tiled)
+    {"dma_128x256", 128, 256, 256},    // 129 .. 256 activation rows in ONE tile: every weight byte is read once
 };
 
 int g_raster_group = 0;  // 0 = per-launch default
@@ -1115,7 +1183,12 @@ hipError_t launch_one(const GemmArgs& a, hipStream_t stream) {
 // of activation rows share them
 template <class E, bool GATED, bool KTAIL, int WP, int WQ, int FP, int FQ>
 void launch_dma_kernel(const dim3 grid, hipStream_t stream, const GemmArgs& a, int tiles_p, int tiles_q, int group) {
-  if constexpr (WP == 2 && WQ == 2 && FP == 2 && FQ == 2) {
+  if constexpr (WP == 2 && WQ == 2 && FP == 2 && (FQ == 2 || FQ == 4)) {  // 128 weight rows x 128 / 256 activation rows
+    if (tiles_q == 1) {  // a single tile of activation rows: three stages (see NS)
+      hipLaunchKernelGGL((tiled_dma_kernel<E, GATED, KTAIL, WP, WQ, FP, FQ, true, 3>), grid, dim3(WP * WQ * 64), 0, stream,
+                         a, tiles_p, tiles_q, group);
+      return;
+    }
     if (tiles_q <= 2) {
       hipLaunchKernelGGL((tiled_dma_kernel<E, GATED, KTAIL, WP, WQ, FP, FQ, true>), grid, dim3(WP * WQ * 64), 0, stream,
                          a, tiles_p, tiles_q, group);
@@ -1232,12 +1305,16 @@ hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
     case 12: return launch_dma<E, GATED, 2, 4, 4, 2>(a, stream);
     case 13: return launch_ring<E, GATED, 5, 2, 2, 4, 4>(a, stream);
     case 14: return launch_ring<E, GATED, 5, 2, 2, 4, 3>(a, stream);
+    case 15: return launch_dma<E, GATED, 2, 2, 2, 4>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
 }  // namespace
 
+#ifndef PLAN_WIDE_TILE
+#define PLAN_WIDE_TILE 1
+#endif
 SplitPlan tiled_split_plan(int np, int nq, int k) {
   const long long t128 = (long long)((np + 127) / 128) * ((nq + 127) / 128);
   const long long t256 = (long long)((np + 255) / 256) * ((nq + 255) / 256);
@@ -1253,7 +1330,17 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
     tiles = t256;
     by_k = k / 1024;
   }
-  int splits = (int)((512 + tiles - 1) / tiles);
+  // One tile of activation rows: three-stage workgroups, one per compute unit, beat two two-stage ones (less
+  // partial-sum traffic as well); 129..256 rows take one 128 x 256 tile per workgroup for the same reason.
+  int target = 512;
+  if (nq <= 128) {
+    target = 256;
+  } else if (nq <= 256 && PLAN_WIDE_TILE) {
+    p.tile = 129;
+    tiles = (np + 127) / 128;
+    target = 256;
+  }
+  int splits = (int)((target + tiles - 1) / tiles);
   if (splits > by_k) splits = by_k;
   if (splits > 16) splits = 16;
   p.splits = splits < 1 ? 1 : splits;
@@ -1287,6 +1374,9 @@ hipError_t launch_splitk_one(const GemmArgs& a, hipStream_t stream) {
 hipError_t launch_tiled_splitk(int dtype, int tile, const GemmArgs& a, hipStream_t stream) {
   if (tile == 128) {
     return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 2>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 2>(a, stream);
+  }
+  if (tile == 129) {  // 128 output features x 256 activation rows
+    return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 4>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 4>(a, stream);
   }
   return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 4, 4>(a, stream) : launch_splitk_one<Fp16, 2, 2, 4, 4>(a, stream);
 }
