@@ -46,11 +46,25 @@ int check_device() {
 // stepping down to 128x128 when a 256-wide grid would leave most of the 256 CUs idle.
 int pick_tiled(int family, int64_t m, int64_t np) {
   const int64_t tiles256 = ((np + 255) / 256) * ((m + 255) / 256);
-  if (tiles256 < 192) {
+  // 256 x 256 tiles down to half-filled compute units. Below that the down product splits K (see
+  // tiled_split_plan); between 129 and 191 tiles one large tile per compute unit beats 128 x 128 tiles in
+  // 1.1 .. 1.4 rounds (down, 4096 x 14336, M = 2304 .. 2816: 250-260 us against 355-365 us; gate/up, 4096 x 22016,
+  // M = 257 .. 512: 79-81 us against 95-102 us).
+  // Up to 128 activation rows are one weight stream whatever the tile count (8192 x 57344, M = 65 .. 128: 173 us on
+  // 128 x 128 tiles, 201-203 us on half-empty large ones).
+  if (tiles256 < 129 || m <= 128) {
     // 128 x 128, direct-to-LDS (with split-K for the down product, see fsw_down). The gate/up product of 129 .. 256
     // activation rows takes them in ONE 128 x 256 tile, so that every weight byte is still read exactly once
     // (4096 x 28672: M = 160: 85 -> 64 us, M = 256: 86 -> 68 us; at M = 128 the 128 x 128 tile is faster, 50 vs 66).
     return (family == 0 && m > 128 && m <= 256) ? 15 : 7;
+  }
+  if (family == 0 && tiles256 > 256 && tiles256 <= 512) {
+    // A few large tiles more than compute units: the second round is nearly empty, while 128 x 128 tiles (two per
+    // compute unit, ~1.3-1.7 x the time per output element) come in rounds a quarter as long. Per round of 256
+    // workgroups: ~33 us against ~75-100 us at K = 4096; the small tile must win by 20 % to be taken. 4096 x 36864,
+    // M = 300 (288 tiles): 151 -> 130 us; 4096 x 22016, M = 640 (258 tiles): 148 -> 119 us.
+    const int64_t tiles128 = ((np + 127) / 128) * ((m + 127) / 128);
+    if (((tiles128 + 255) / 256) * 44 < ((tiles256 + 255) / 256) * 100) return 7;
   }
   // 256 x 256: the gate/up product runs best on the four-stage ring, the deep-K down product on two stages
   return family == 0 ? 8 : 5;

@@ -1154,7 +1154,7 @@ const TiledVariant kVariants[] = {
     {"ring8w_256x256_b", 256, 256, 512},  // 8 waves, wave tile 64 x 128
     {"dma8w_256x256", 256, 256, 512},
     {"ring5_256x256", 256, 256, 256},  // five-stage ring: all 160 KB of LDS, four K tiles in flight
-    {"ring5_256x192", 256, 192, 256},  // 192 activation rows: fewer padded rows / idle CUs for some M (see pick_tiled)
+    {"ring5_256x192", 256, 192, 256},  // 192 activation rows: within 5 % of the default either way, not dispatched
     {"dma_128x256", 128, 256, 256},    // 129 .. 256 activation rows in ONE tile: every weight byte is read once
 };
 
@@ -1319,7 +1319,7 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
   const long long t128 = (long long)((np + 127) / 128) * ((nq + 127) / 128);
   const long long t256 = (long long)((np + 255) / 256) * ((nq + 255) / 256);
   SplitPlan p = {256, 1};
-  if (t128 <= 0 || t256 >= 192) return p;
+  if (t128 <= 0 || t256 > 128) return p;  // more large tiles than half the compute units: no split (see pick_tiled)
   int by_k;
   long long tiles;
   if (t128 < 256) {
@@ -1329,6 +1329,42 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
   } else {
     tiles = t256;
     by_k = k / 1024;
+  }
+  if (nq > 256) {
+    // Several tiles of activation rows: all workgroups should be resident at once (two 128 x 128 workgroups or one
+    // 256 x 256 workgroup per compute unit: a second, partly filled round costs a whole one; 640 rows of 4096 x
+    // 14336: 160 tiles x 3 splits 86 us, x 4 splits 110 us), and every split adds a partial tile to write and read
+    // back. Estimated time per candidate, in us on 256 compute units: MFMA work of the busiest compute unit at
+    // ~5.1 TFLOP/s (a lone 128 x 128 workgroup runs at half of that, the small tile costs ~15 % more per flop) plus
+    // the fp32 partials at ~5 TB/s. Measured against it (4096 x 14336): 257 rows 128/4 60 us, 1024 rows 256/4
+    // 119 us, 2048 rows 256/2 214 us, each the fastest of 15 tile/split pairs tried.
+    const int nkt = (k + 63) / 64;
+    double best = 0.0;
+    p.tile = 128;
+    p.splits = 1;
+    for (int c = 0; c < 2; ++c) {
+      const int tile = c == 0 ? 128 : 256;
+      const long long nt = c == 0 ? t128 : t256;
+      const long long slots = c == 0 ? 512 : 256;
+      long long smax = slots / nt;
+      const long long deep = c == 0 ? k / 512 : k / 1024;  // at least 8 (16) K tiles of 64 per partition
+      if (smax > deep) smax = deep;
+      if (smax > 16) smax = 16;
+      if (smax < 1) smax = 1;
+      for (int sp = 1; sp <= (int)smax; ++sp) {
+        const double kper = 64.0 * ((nkt + sp - 1) / sp);
+        const double rounds = (double)((nt * sp + slots - 1) / slots);
+        const double mfma = 2.0 * kper * tile * tile * (c == 0 ? 2.0 * 1.15 : 1.0) * rounds / 5.1e6;
+        const double partials = sp > 1 ? 8.0 * sp * (double)nq * (double)np / 5.0e6 : 0.0;
+        if (best == 0.0 || mfma + partials < best) {
+          best = mfma + partials;
+          p.tile = tile;
+          p.splits = sp;
+        }
+      }
+    }
+    if (p.splits == 1) p.tile = 128;  // unsplit mid-size problems keep the smaller tile
+    return p;
   }
   // One tile of activation rows: three-stage workgroups, one per compute unit, beat two two-stage ones (less
   // partial-sum traffic as well); 129..256 rows take one 128 x 256 tile per workgroup for the same reason.

@@ -554,7 +554,7 @@ def test_large_tiles_on_row_major_activations(capi):
     fsw_down without the optional scratch for a blocked copy of H. Both against the oracle, and the down projection
     bit for bit against the call that does get the scratch."""
     L = capi.lib()
-    M, d, ff = 600, 520, 12800           # 3 x 100 tiles of 256 x 256, K = 520 is not a multiple of 64
+    M, d, ff = 1000, 520, 12800          # 4 x 100 tiles of 256 x 256, K = 520 is not a multiple of 64
     assert capi.variant_name(0, 0, M, 2 * ff, d) == "pair16_256x256" and L.fsw_gateup_workspace_bytes(0, M, 2 * ff, d) == 0
     inp = fsw_weights.make_inputs(M, d, ff, torch.bfloat16, seed=31, x_scale=0.5)
     g = to_dev(inp)
