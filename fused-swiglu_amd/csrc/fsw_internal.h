@@ -45,6 +45,7 @@ hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, h
 int raster_group(bool gated);  // activation-row tiles per raster band of the tiled kernels
 // the 16x16x32 pair-ring kernel (kernels_pair16.hip) for GemmArgs::layout 0, 1, 3, 5, 7
 hipError_t launch_pair16(int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
+hipError_t launch_pair16_splitk(int dtype, const GemmArgs& a, hipStream_t stream);  // partials only, no reduction
 int pair_ring_mode();  // kernel family behind the 256 x 256 tiles: 2 = 16x16x32 pair ring, 1 / 0 = 32x32x16 kernels
 hipError_t launch_tiled_blocked(int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
 // row-major [rows, k] (row stride ld elements) -> blocked; gated_order: W13's up/gate rows de-interleaved per panel

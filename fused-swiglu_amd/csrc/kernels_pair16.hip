@@ -37,9 +37,21 @@ typedef __attribute__((address_space(3))) void lds_void;
 // of the pair slots (128 KB of LDS).
 // QROW: the activation operand is row-major (callers without scratch for a blocked copy; few ragged activation
 // panels, where re-blocking does not pay): 64-byte requests per row and K tile, rows past nq read as zero.
-template <class E, bool GATED, bool KTAIL, bool OBLK, bool PBLK = false, bool QROW = false>
+// SPLIT (row-major operands, plain product): blockIdx.y selects one of a.splits contiguous runs of 64-element K
+// pairs; the workgroup multiplies that run only and stores its fp32 accumulators to a.partial[blockIdx.y][nq][np].
+template <class E, bool GATED, bool KTAIL, bool OBLK, bool PBLK = false, bool QROW = false, bool SPLIT = false>
 __global__ void __launch_bounds__(256)
-tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const int group) {
+tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, const int group) {
+  static_assert(!SPLIT || (QROW && !GATED && !OBLK && !PBLK), "split-K: row-major operands, plain product");
+  GemmArgs a = a_in;
+  if constexpr (SPLIT) {  // the run of this workgroup as a product of its own: shifted operands, shorter K
+    const int per = ((a_in.k + 63) / 64 + a_in.splits - 1) / a_in.splits * 64;
+    const long long k0 = (long long)blockIdx.y * per;
+    const long long left = a_in.k - k0;
+    a.k = left < 0 ? 0 : (left < per ? (int)left : per);
+    a.P = (const unsigned short*)a_in.P + k0;
+    a.Q = (const unsigned short*)a_in.Q + k0;
+  }
   constexpr int WP = 2, WQ = 2;
   constexpr int NB = 8;  // 16-row blocks per wave and operand
   constexpr int BP = 256, BQ = 256;
@@ -322,6 +334,26 @@ tiled_pair16_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, cons
         }
       }
     }
+  } else if constexpr (SPLIT) {
+    float* const part = a.partial + (long long)blockIdx.y * a.nq * a.np;
+    const bool vec_ok = (a.np & 3) == 0;
+#pragma unroll
+    for (int g = 0; g < NB; ++g) {
+      const int m = q0 + wq * 128 + g * 16 + r16;
+      if (m >= a.nq) continue;
+      float* prow = part + (long long)m * a.np;
+#pragma unroll
+      for (int f = 0; f < NB; ++f) {
+        const int n = p0 + wp * 128 + f * 16 + c4 * 4;
+        if (vec_ok && n + 3 < a.np) {
+          *(f32x4*)(prow + n) = acc[f][g];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < a.np) prow[n + e] = acc[f][g][e];
+        }
+      }
+    }
   } else {
     unsigned short* O = (unsigned short*)a.O;
     constexpr int FO = GATED ? NB / 2 : NB;
@@ -387,6 +419,23 @@ hipError_t launch_pair16_rowmajor(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// both operands row-major, plain product, K split over blockIdx.y: fp32 partial tiles to a.partial
+template <class E>
+hipError_t launch_pair16_split(const GemmArgs& a, hipStream_t stream) {
+  const int tiles_p = (a.np + 255) / 256;
+  const int tiles_q = (a.nq + 255) / 256;
+  if (tiles_p <= 0 || tiles_q <= 0 || a.splits <= 0) return hipSuccess;
+  const dim3 grid((unsigned)(tiles_p * tiles_q), (unsigned)a.splits), block(256);
+  if (a.k % 64 == 0) {
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, false, false, false, false, true, true>), grid, block, 0, stream, a,
+                       tiles_p, tiles_q, raster_group(false));
+  } else {
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, false, true, false, false, true, true>), grid, block, 0, stream, a,
+                       tiles_p, tiles_q, raster_group(false));
+  }
+  return hipGetLastError();
+}
+
 // both operands blocked (prepacked weights): the 16x16x32 kernel with a stage ring for the weights
 template <class E, bool GATED, bool OBLK>
 hipError_t launch_pair16_blocked_xw(const GemmArgs& a, hipStream_t stream) {
@@ -415,6 +464,11 @@ hipError_t launch_pair16_typed(bool gated, const GemmArgs& a, hipStream_t stream
 // GemmArgs::layout: bit 0 = activations blocked, bit 1 = output blocked (gated only), bit 2 = weights blocked
 hipError_t launch_pair16(int dtype, bool gated, const GemmArgs& a, hipStream_t stream) {
   return dtype == 0 ? launch_pair16_typed<Bf16>(gated, a, stream) : launch_pair16_typed<Fp16>(gated, a, stream);
+}
+
+// Row-major plain product with K split over a.splits workgroups per tile; fp32 partials to a.partial (not reduced).
+hipError_t launch_pair16_splitk(int dtype, const GemmArgs& a, hipStream_t stream) {
+  return dtype == 0 ? launch_pair16_split<Bf16>(a, stream) : launch_pair16_split<Fp16>(a, stream);
 }
 
 }  // namespace fsw

@@ -1385,6 +1385,14 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
 }
 
 namespace {
+template <class E>
+hipError_t launch_splitk_reduce(const GemmArgs& a, hipStream_t stream) {
+  const long long work = (long long)a.nq * ((a.np + 3) / 4);
+  hipLaunchKernelGGL((splitk_reduce_kernel<E>), dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, a.partial,
+                     a.splits, a.nq, a.np, (unsigned short*)a.O, a.ldo);
+  return hipGetLastError();
+}
+
 template <class E, int WP, int WQ, int FP, int FQ>
 hipError_t launch_splitk_one(const GemmArgs& a, hipStream_t stream) {
   constexpr int BP = WP * FP * 32, BQ = WQ * FQ * 32;
@@ -1400,10 +1408,7 @@ hipError_t launch_splitk_one(const GemmArgs& a, hipStream_t stream) {
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || a.splits <= 1) return e;
-  const long long work = (long long)a.nq * ((a.np + 3) / 4);
-  hipLaunchKernelGGL((splitk_reduce_kernel<E>), dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, a.partial,
-                     a.splits, a.nq, a.np, (unsigned short*)a.O, a.ldo);
-  return hipGetLastError();
+  return launch_splitk_reduce<E>(a, stream);
 }
 }  // namespace
 
@@ -1413,6 +1418,11 @@ hipError_t launch_tiled_splitk(int dtype, int tile, const GemmArgs& a, hipStream
   }
   if (tile == 129) {  // 128 output features x 256 activation rows
     return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 4>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 4>(a, stream);
+  }
+  if (g_pair_ring == 2 && a.splits > 1) {  // 256 x 256 on the 16x16x32 kernel
+    const hipError_t e = launch_pair16_splitk(dtype, a, stream);
+    if (e != hipSuccess) return e;
+    return dtype == 0 ? launch_splitk_reduce<Bf16>(a, stream) : launch_splitk_reduce<Fp16>(a, stream);
   }
   return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 4, 4>(a, stream) : launch_splitk_one<Fp16, 2, 2, 4, 4>(a, stream);
 }
