@@ -1335,9 +1335,10 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
     // 256 x 256 workgroup per compute unit: a second, partly filled round costs a whole one; 640 rows of 4096 x
     // 14336: 160 tiles x 3 splits 86 us, x 4 splits 110 us), and every split adds a partial tile to write and read
     // back. Estimated time per candidate, in us on 256 compute units: MFMA work of the busiest compute unit at
-    // ~5.1 TFLOP/s (a lone 128 x 128 workgroup runs at half of that, the small tile costs ~15 % more per flop) plus
-    // the fp32 partials at ~5 TB/s. Measured against it (4096 x 14336): 257 rows 128/4 60 us, 1024 rows 256/4
-    // 119 us, 2048 rows 256/2 214 us, each the fastest of 15 tile/split pairs tried.
+    // ~5.1 TFLOP/s (a lone 128 x 128 workgroup runs at half of that, the small tile costs ~15 % more per flop, the
+    // large one on 16x16x32 MFMAs ~15 % less) plus the fp32 partials at ~5 TB/s. Measured against it (4096 x 14336):
+    // 257 rows 128/5 59 us, 640 rows 128/3 85 us, 1024 rows 256/4 106 us, 2048 rows 256/2 185 us, each within 5 % of
+    // the fastest of 12 tile/split pairs tried.
     const int nkt = (k + 63) / 64;
     double best = 0.0;
     p.tile = 128;
@@ -1354,7 +1355,7 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
       for (int sp = 1; sp <= (int)smax; ++sp) {
         const double kper = 64.0 * ((nkt + sp - 1) / sp);
         const double rounds = (double)((nt * sp + slots - 1) / slots);
-        const double mfma = 2.0 * kper * tile * tile * (c == 0 ? 2.0 * 1.15 : 1.0) * rounds / 5.1e6;
+        const double mfma = 2.0 * kper * tile * tile * (c == 0 ? 2.0 * 1.15 : 0.85) * rounds / 5.1e6;
         const double partials = sp > 1 ? 8.0 * sp * (double)nq * (double)np / 5.0e6 : 0.0;
         if (best == 0.0 || mfma + partials < best) {
           best = mfma + partials;
