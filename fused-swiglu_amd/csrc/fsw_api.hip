@@ -139,13 +139,23 @@ int fsw_set_variant(int family, int variant) {
   return FSW_OK;
 }
 
+static bool down_reblock_wanted(int64_t M, int64_t D, int64_t FF);
+
 const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, int64_t K_or_FF) {
   (void)dtype;
-  (void)K_or_FF;
   if (family < 0 || family > 1) return "invalid";
   const int v = resolve_variant(family, M, N_or_D);
   if (v == VARIANT_SKINNY) return decode_stream_wanted(family, M, N_or_D, K_or_FF) ? "decode_stream" : "skinny";
   if ((v == 8 || v == 5) && g_forced_variant[family] < 0 && fsw::pair_ring_mode() == 2) return "pair16_256x256";
+  if (family == 1 && g_forced_variant[1] < 0 && !down_reblock_wanted(M, N_or_D, K_or_FF) && M <= MAX_DIM &&
+      N_or_D > 0 && N_or_D <= MAX_DIM && K_or_FF > 0 && K_or_FF <= MAX_DIM) {
+    const fsw::SplitPlan plan = fsw::tiled_split_plan((int)N_or_D, (int)M, (int)K_or_FF);
+    if (plan.splits > 1) {
+      if (plan.tile == 128) return "splitk_dma_128x128";
+      if (plan.tile == 129) return "splitk_dma_128x256";
+      return fsw::pair_ring_mode() == 2 ? "splitk_pair16_256x256" : "splitk_dma_256x256";
+    }
+  }
   return fsw::tiled_variant(v).name;
 }
 

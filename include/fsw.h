@@ -160,7 +160,8 @@ FSW_API int fsw_version(void);
  */
 FSW_API int fsw_set_variant(int family, int variant);
 
-/* Name of the kernel variant the dispatcher picks for this shape (static storage). */
+/* Name of the kernel variant the dispatcher picks for this shape (static storage); "splitk_<kernel>" when the
+ * down projection splits K (family 1; K_or_FF decides). */
 FSW_API const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, int64_t K_or_FF);
 
 #ifdef __cplusplus

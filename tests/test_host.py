@@ -122,7 +122,13 @@ def test_variant_choice_by_regime(capi):
         L.fsw_set_variant(1, -1)
     # the down product with few output tiles and a deep K asks for split-K scratch; large or tiny M does not
     ws = capi.lib().fsw_down_workspace_bytes
-    assert ws(0, 256, 4096, 14336) == 8 * 256 * 4096 * 4
+    assert ws(0, 256, 4096, 14336) == 8 * 256 * 4096 * 4 and name(1, 256, 4096, 14336) == "splitk_dma_128x256"
+    assert name(1, 128, 4096, 14336) == "splitk_dma_128x128" and ws(0, 128, 4096, 14336) == 8 * 128 * 4096 * 4
+    # above 256 rows: as many splits as keep all workgroups resident at once, on the tile the time estimate favours
+    assert name(1, 640, 4096, 14336) == "splitk_dma_128x128" and ws(0, 640, 4096, 14336) == 3 * 640 * 4096 * 4
+    assert name(1, 1024, 4096, 14336) == "splitk_pair16_256x256" and ws(0, 1024, 4096, 14336) == 4 * 1024 * 4096 * 4
+    assert name(1, 2048, 4096, 14336) == "splitk_pair16_256x256" and ws(0, 2048, 4096, 14336) == 2 * 2048 * 4096 * 4
+    assert name(1, 2304, 4096, 14336) == "pair16_256x256"    # more than 128 large tiles: no split
     # large-tile regime: scratch for a blocked copy of H (optional: without it fsw_down runs on row-major H)
     assert ws(0, 8192, 4096, 14336) == L.fsw_blocked_bytes(8192, 14336) == 8192 * 14336 * 2
     assert ws(0, 3000, 4096, 14336) == L.fsw_blocked_bytes(3000, 14336) and ws(0, 16, 4096, 14336) == 0
