@@ -11,6 +11,8 @@ printed and optionally written as CSV.
 
   python bench_swiglu.py                         # full sweep
   python bench_swiglu.py --tokens 512 4096 --csv results.csv
+  python bench_swiglu.py --forward --k 4096 --n 28672 --tokens 128 1024   # also the whole MLP forward (with the
+                                                 # down projection [K, N/2]) against mm + eager gating + mm
 """
 import argparse
 import sys
@@ -55,7 +57,7 @@ def timed(fn, flush, warmup_ms=25.0, rep_ms=100.0):
     return q[0].item(), q[1].item(), q[2].item()
 
 
-def run(tokens, k=K_DEFAULT, n=N_DEFAULT, device="cuda:0", out=sys.stdout, csv=None):
+def run(tokens, k=K_DEFAULT, n=N_DEFAULT, device="cuda:0", out=sys.stdout, csv=None, forward=False):
     import fused_mlp_module
     flush = torch.empty(512 << 20, dtype=torch.uint8, device=device)
     rows = []
@@ -74,9 +76,24 @@ def run(tokens, k=K_DEFAULT, n=N_DEFAULT, device="cuda:0", out=sys.stdout, csv=N
             torch.mm(a, bt, out=c2)
             return c2[:, : n // 2] * F.silu(c2[:, n // 2:])
 
-        for name, fn in (("hipBLASLt+eager", library_plus_eager), ("Fused", fused)):
+        legs = [("hipBLASLt+eager", library_plus_eager, reference_flops(m, n, k)), ("Fused", fused, reference_flops(m, n, k))]
+        if forward:
+            w2 = torch.randn((k, n // 2), dtype=torch.bfloat16, device=device) / (n // 2) ** 0.5
+            w2t = w2.T
+            y = torch.empty((m, k), dtype=torch.bfloat16, device=device)
+            fwd_flops = reference_flops(m, n, k) + m * k * (n - 1)
+
+            def fused_forward():
+                return fused_mlp_module.fused_swiglu_mlp_bf16(a, b, w2)
+
+            def library_forward():
+                torch.mm(a, bt, out=c2)
+                return torch.mm(c2[:, : n // 2] * F.silu(c2[:, n // 2:]), w2t, out=y)
+
+            legs += [("hipBLASLt forward", library_forward, fwd_flops), ("Fused forward", fused_forward, fwd_flops)]
+        for name, fn, flops in legs:
             ms, lo, hi = timed(fn, flush)
-            tf = lambda t: reference_flops(m, n, k) * 1e-12 / (t * 1e-3)
+            tf = lambda t: flops * 1e-12 / (t * 1e-3)
             rows.append((m, name, ms, tf(ms), tf(hi), tf(lo)))
             print("%8d | %-18s | %10.4f | %10.1f | %10.1f | %10.1f" % rows[-1], file=out)
         del a, b, c, c2, bt
@@ -94,10 +111,11 @@ def main(argv=None):
     ap.add_argument("--k", type=int, default=K_DEFAULT)
     ap.add_argument("--n", type=int, default=N_DEFAULT, help="full N = 2 * ff")
     ap.add_argument("--csv", default=None)
+    ap.add_argument("--forward", action="store_true", help="also time the whole forward, down projection included")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         sys.exit("bench_swiglu.py needs the GPU: the extension has no CPU path")
-    run(args.tokens, args.k, args.n, csv=args.csv)
+    run(args.tokens, args.k, args.n, csv=args.csv, forward=args.forward)
 
 
 if __name__ == "__main__":

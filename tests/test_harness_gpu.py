@@ -43,3 +43,6 @@ def test_benchmark_sweep_small(ext, tmp_path):
     for r in rows:
         assert r[2] > 0 and r[4] <= r[3] <= r[5]
     assert csv.read_text().startswith("Tokens,provider,ms,tflops")
+    rows = bench_swiglu.run([128], k=1024, n=2048, out=io.StringIO(), forward=True)
+    assert [r[1] for r in rows] == ["hipBLASLt+eager", "Fused", "hipBLASLt forward", "Fused forward"]
+    assert all(r[2] > 0 for r in rows)
