@@ -55,8 +55,10 @@ int pick_tiled(int family, int64_t m, int64_t np) {
   if (tiles256 < 129 || m <= 128) {
     // 128 x 128, direct-to-LDS (with split-K for the down product, see fsw_down). The gate/up product of 129 .. 256
     // activation rows takes them in ONE 128 x 256 tile, so that every weight byte is still read exactly once
-    // (4096 x 28672: M = 160: 85 -> 64 us, M = 256: 86 -> 68 us; at M = 128 the 128 x 128 tile is faster, 50 vs 66).
-    return (family == 0 && m > 128 && m <= 256) ? 15 : 7;
+    // (4096 x 28672: M = 160: 85 -> 64 us, M = 256: 86 -> 68 us; at M = 128 the 128 x 128 tile is faster, 50 vs 66),
+    // provided those tiles still cover half the compute units (1024 x 5632 at M = 256: 44 of them, 18.5 us against
+    // 10.5 us for 88 tiles of 128 x 128).
+    return (family == 0 && m > 128 && m <= 256 && (np + 127) / 128 >= 128) ? 15 : 7;
   }
   if (family == 0 && tiles256 > 256 && tiles256 <= 512) {
     // A few large tiles more than compute units: the second round is nearly empty, while 128 x 128 tiles (two per
