@@ -148,9 +148,8 @@ const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, i
   if (family < 0 || family > 1) return "invalid";
   const int v = resolve_variant(family, M, N_or_D);
   if (v == VARIANT_SKINNY) return decode_stream_wanted(family, M, N_or_D, K_or_FF) ? "decode_stream" : "skinny";
-  if ((v == 8 || v == 5) && g_forced_variant[family] < 0 && fsw::pair_ring_mode() == 2) return "pair16_256x256";
-  if (family == 1 && g_forced_variant[1] < 0 && !down_reblock_wanted(M, N_or_D, K_or_FF) && M <= MAX_DIM &&
-      N_or_D > 0 && N_or_D <= MAX_DIM && K_or_FF > 0 && K_or_FF <= MAX_DIM) {
+  if (family == 1 && g_forced_variant[1] < 0 && M <= MAX_DIM && N_or_D > 0 && N_or_D <= MAX_DIM && K_or_FF > 0 &&
+      K_or_FF <= MAX_DIM) {
     const fsw::SplitPlan plan = fsw::tiled_split_plan((int)N_or_D, (int)M, (int)K_or_FF);
     if (plan.splits > 1) {
       if (plan.tile == 128) return "splitk_dma_128x128";
@@ -158,6 +157,7 @@ const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, i
       return fsw::pair_ring_mode() == 2 ? "splitk_pair16_256x256" : "splitk_dma_256x256";
     }
   }
+  if ((v == 8 || v == 5) && g_forced_variant[family] < 0 && fsw::pair_ring_mode() == 2) return "pair16_256x256";
   return fsw::tiled_variant(v).name;
 }
 
@@ -239,6 +239,7 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
 // two-stage kernel on row-major H). Same rule for ragged panel counts as fsw_gateup_workspace_bytes.
 static bool down_reblock_wanted(int64_t M, int64_t D, int64_t FF) {
   if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[1] >= 0 || pick_tiled(1, M, D) != 5) return false;
+  if (M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM || fsw::tiled_split_plan((int)D, (int)M, (int)FF).splits > 1) return false;
   return M >= 1024 || M % 256 == 0;
 }
 
@@ -313,7 +314,9 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
 // and H never exists row-major (the gate/up epilogue writes it blocked, the down projection reads it blocked).
 static bool blocked_regime(int64_t M, int64_t D, int64_t FF) {
   if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[0] >= 0 || g_forced_variant[1] >= 0) return false;
-  return pick_tiled(0, M, 2 * FF) == 8 && pick_tiled(1, M, D) == 5;
+  if (M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM / 2) return false;
+  return pick_tiled(0, M, 2 * FF) == 8 && pick_tiled(1, M, D) == 5 &&
+         fsw::tiled_split_plan((int)D, (int)M, (int)FF).splits == 1;  // a split-K down projection reads row-major H
 }
 
 size_t fsw_blocked_bytes(int64_t rows, int64_t k) {

@@ -1319,7 +1319,10 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
   const long long t128 = (long long)((np + 127) / 128) * ((nq + 127) / 128);
   const long long t256 = (long long)((np + 255) / 256) * ((nq + 255) / 256);
   SplitPlan p = {256, 1};
-  if (t128 <= 0 || t256 > 128) return p;  // more large tiles than half the compute units: no split (see pick_tiled)
+  // One or two activation tiles with more large tiles than half the compute units: no split (see pick_tiled).
+  // More rows: splitting can still pay by evening out rounds (288 tiles are two rounds of K, 288 x 3 are four
+  // rounds of K / 3), up to 512 tiles.
+  if (t128 <= 0 || t256 > (nq > 256 ? 512 : 128)) return p;
   int by_k;
   long long tiles;
   if (t128 < 256) {
@@ -1339,24 +1342,34 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
     // large one on 16x16x32 MFMAs ~15 % less) plus the fp32 partials at ~5 TB/s. Measured against it (4096 x 14336):
     // 257 rows 128/5 59 us, 640 rows 128/3 85 us, 1024 rows 256/4 106 us, 2048 rows 256/2 185 us, each within 5 % of
     // the fastest of 12 tile/split pairs tried.
+    // From 129 large tiles up the unsplit alternative is the 16x16x32 kernel on blocked H (~8 % faster than on
+    // row-major H, which the split kernel reads): there only large-tile splits are candidates, over several rounds
+    // if need be, they must win by 15 %, and their partials stay under 256 MB.
     const int nkt = (k + 63) / 64;
-    double best = 0.0;
+    const bool large = t256 >= 129;
+    double best = 0.0, unsplit = 0.0;
     p.tile = 128;
     p.splits = 1;
-    for (int c = 0; c < 2; ++c) {
+    for (int c = large ? 1 : 0; c < 2; ++c) {
       const int tile = c == 0 ? 128 : 256;
       const long long nt = c == 0 ? t128 : t256;
       const long long slots = c == 0 ? 512 : 256;
-      long long smax = slots / nt;
+      long long smax = large ? 16 : slots / nt;
       const long long deep = c == 0 ? k / 512 : k / 1024;  // at least 8 (16) K tiles of 64 per partition
       if (smax > deep) smax = deep;
       if (smax > 16) smax = 16;
       if (smax < 1) smax = 1;
       for (int sp = 1; sp <= (int)smax; ++sp) {
+        if (sp > 1 && 4.0 * sp * (double)nq * (double)np > 256e6) break;
         const double kper = 64.0 * ((nkt + sp - 1) / sp);
-        const double rounds = (double)((nt * sp + slots - 1) / slots);
+        // a partly filled round of large tiles runs at a higher clock: 0.6 .. 0.95 of a full one (4096 x 14336:
+        // 16 tiles 0.57, 144 tiles 0.80, 176 tiles 0.83 of the 310 us a round of 256 takes)
+        const long long wgs = nt * sp;
+        const double rounds = c == 0 ? (double)((wgs + slots - 1) / slots)
+                                     : (double)(wgs / slots) + (wgs % slots ? 0.6 + 0.35 * (wgs % slots) / slots : 0.0);
         const double mfma = 2.0 * kper * tile * tile * (c == 0 ? 2.0 * 1.15 : 0.85) * rounds / 5.1e6;
         const double partials = sp > 1 ? 8.0 * sp * (double)nq * (double)np / 5.0e6 : 0.0;
+        if (sp == 1 && c == 1) unsplit = mfma;
         if (best == 0.0 || mfma + partials < best) {
           best = mfma + partials;
           p.tile = tile;
@@ -1364,7 +1377,8 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
         }
       }
     }
-    if (p.splits == 1) p.tile = 128;  // unsplit mid-size problems keep the smaller tile
+    if (large && p.splits > 1 && best > 0.85 * unsplit) p.splits = 1;
+    if (p.splits == 1) p.tile = large ? 256 : 128;  // unsplit mid-size problems keep the smaller tile
     return p;
   }
   // One tile of activation rows: three-stage workgroups, one per compute unit, beat two two-stage ones (less

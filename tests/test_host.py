@@ -125,10 +125,12 @@ def test_variant_choice_by_regime(capi):
     assert ws(0, 256, 4096, 14336) == 8 * 256 * 4096 * 4 and name(1, 256, 4096, 14336) == "splitk_dma_128x256"
     assert name(1, 128, 4096, 14336) == "splitk_dma_128x128" and ws(0, 128, 4096, 14336) == 8 * 128 * 4096 * 4
     # above 256 rows: as many splits as keep all workgroups resident at once, on the tile the time estimate favours
-    assert name(1, 640, 4096, 14336) == "splitk_dma_128x128" and ws(0, 640, 4096, 14336) == 3 * 640 * 4096 * 4
+    assert name(1, 257, 4096, 14336) == "splitk_dma_128x128" and ws(0, 257, 4096, 14336) == 5 * 257 * 4096 * 4
     assert name(1, 1024, 4096, 14336) == "splitk_pair16_256x256" and ws(0, 1024, 4096, 14336) == 4 * 1024 * 4096 * 4
     assert name(1, 2048, 4096, 14336) == "splitk_pair16_256x256" and ws(0, 2048, 4096, 14336) == 2 * 2048 * 4096 * 4
-    assert name(1, 2304, 4096, 14336) == "pair16_256x256"    # more than 128 large tiles: no split
+    assert name(1, 2304, 4096, 14336) == "pair16_256x256"    # 144 large tiles in one round: no split
+    # 288 large tiles of a very deep K: three splits (four rounds of K / 3 instead of two of K), H stays row-major
+    assert name(1, 2049, 8192, 28672) == "splitk_pair16_256x256" and ws(0, 2049, 8192, 28672) == 3 * 2049 * 8192 * 4
     # large-tile regime: scratch for a blocked copy of H (optional: without it fsw_down runs on row-major H)
     assert ws(0, 8192, 4096, 14336) == L.fsw_blocked_bytes(8192, 14336) == 8192 * 14336 * 2
     assert ws(0, 3000, 4096, 14336) == L.fsw_blocked_bytes(3000, 14336) and ws(0, 16, 4096, 14336) == 0

@@ -215,8 +215,8 @@ def test_split_k_down_projection(capi, dtype):
     workspace, then one rounding). Checked against the oracle and, bit for bit up to summation order, against the
     unsplit kernel."""
     L = capi.lib()
-    # the last three shapes are planned on 256 x 256 tiles (5, 5 and 3 splits; the last two with a K tail, the last
-    # with ragged M and d as well), the others on 128 x 128 or 128 x 256
+    # the last three shapes are planned on 256 x 256 tiles (the last two with a K tail, the last with ragged M and d
+    # as well), the others on 128 x 128 or 128 x 256
     for (M, d, ff) in [(200, 512, 4096), (130, 520, 2120), (65, 136, 8192), (256, 1024, 14336), (300, 264, 1032), (1024, 1024, 4096), (700, 2048, 2056), (768, 4096, 8192),
                        (768, 4096, 8200), (1300, 3080, 8200)]:
         inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=900 + M, x_scale=0.5)
