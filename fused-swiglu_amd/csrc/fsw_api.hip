@@ -58,7 +58,10 @@ int pick_tiled(int family, int64_t m, int64_t np) {
     // (4096 x 28672: M = 160: 85 -> 64 us, M = 256: 86 -> 68 us; at M = 128 the 128 x 128 tile is faster, 50 vs 66),
     // provided those tiles still cover half the compute units (1024 x 5632 at M = 256: 44 of them, 18.5 us against
     // 10.5 us for 88 tiles of 128 x 128).
-    return (family == 0 && m > 128 && m <= 256 && (np + 127) / 128 >= 128) ? 15 : 7;
+    // Up to 192 rows the tile is 128 x 192: the single-tile kernels are bound by their MFMA and LDS work as much as
+    // by the weight stream (4096 x 28672, M = 160: 65 -> 54 us; 5120 x 27648: 89 -> 68 us).
+    if (family == 0 && m > 128 && m <= 256 && (np + 127) / 128 >= 128) return m <= 192 ? 16 : 15;
+    return 7;
   }
   if (family == 0 && tiles256 > 256 && tiles256 <= 512) {
     // A few large tiles more than compute units: the second round is nearly empty, while 128 x 128 tiles (two per
@@ -154,6 +157,7 @@ const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, i
     if (plan.splits > 1) {
       if (plan.tile == 128) return "splitk_dma_128x128";
       if (plan.tile == 129) return "splitk_dma_128x256";
+      if (plan.tile == 130) return "splitk_dma_128x192";
       return fsw::pair_ring_mode() == 2 ? "splitk_pair16_256x256" : "splitk_dma_256x256";
     }
   }

@@ -55,7 +55,7 @@ hipError_t launch_block_rows(const void* src, long long ld, int rows, int k, voi
 // tile (128 or 256 square) and how many K partitions, so that about two workgroups per CU are in flight.
 // splits == 1 means the ordinary launch path.
 struct SplitPlan {
-  int tile;    // 128 or 256 (square), or 129 = 128 output features x 256 activation rows
+  int tile;    // 128 or 256 (square), 129 = 128 output features x 256 activation rows, 130 = 128 x 192
   int splits;  // K partitions
 };
 SplitPlan tiled_split_plan(int np, int nq, int k);

@@ -1156,6 +1156,7 @@ const TiledVariant kVariants[] = {
     {"ring5_256x256", 256, 256, 256},  // five-stage ring: all 160 KB of LDS, four K tiles in flight
     {"ring5_256x192", 256, 192, 256},  // 192 activation rows: within 5 % of the default either way, not dispatched
     {"dma_128x256", 128, 256, 256},    // 129 .. 256 activation rows in ONE tile: every weight byte is read once
+    {"dma_128x192", 128, 192, 256},    // the same for 129 .. 192 rows
 };
 
 int g_raster_group = 0;  // 0 = per-launch default
@@ -1183,11 +1184,11 @@ hipError_t launch_one(const GemmArgs& a, hipStream_t stream) {
 // of activation rows share them
 template <class E, bool GATED, bool KTAIL, int WP, int WQ, int FP, int FQ>
 void launch_dma_kernel(const dim3 grid, hipStream_t stream, const GemmArgs& a, int tiles_p, int tiles_q, int group) {
-  if constexpr (WP == 2 && WQ == 2 && FP == 2 && (FQ == 2 || FQ == 4)) {  // 128 weight rows x 128 / 256 activation rows
+  if constexpr (WP == 2 && WQ == 2 && FP == 2 && FQ >= 2 && FQ <= 4) {  // 128 weight rows x 128 / 192 / 256 activation rows
     // a single tile of activation rows: three stages (see NS). They leave room for one workgroup per compute unit,
     // so 128 x 128 launches of more than 256 workgroups keep two stages and two workgroups (8192 x 57344 at 65 rows,
     // 448 workgroups: 168 -> 158 us)
-    if (tiles_q == 1 && (FQ == 4 || (long long)grid.x * grid.y <= 256)) {
+    if (tiles_q == 1 && (FQ >= 3 || (long long)grid.x * grid.y <= 256)) {
       hipLaunchKernelGGL((tiled_dma_kernel<E, GATED, KTAIL, WP, WQ, FP, FQ, true, 3>), grid, dim3(WP * WQ * 64), 0, stream,
                          a, tiles_p, tiles_q, group);
       return;
@@ -1309,6 +1310,7 @@ hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
     case 13: return launch_ring<E, GATED, 5, 2, 2, 4, 4>(a, stream);
     case 14: return launch_ring<E, GATED, 5, 2, 2, 4, 3>(a, stream);
     case 15: return launch_dma<E, GATED, 2, 2, 2, 4>(a, stream);
+    case 16: return launch_dma<E, GATED, 2, 2, 2, 3>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -1394,7 +1396,7 @@ SplitPlan tiled_split_plan(int np, int nq, int k) {
     if (sw > by_k) sw = by_k;
     if (sw > 16) sw = 16;
     if (wide * sw >= 192) {
-      p.tile = 129;
+      p.tile = nq <= 192 ? 130 : 129;  // 128 x 192 does a quarter less MFMA work where 192 rows are enough
       tiles = wide;
       target = 256;
     }
@@ -1440,6 +1442,9 @@ hipError_t launch_splitk_one(const GemmArgs& a, hipStream_t stream) {
 hipError_t launch_tiled_splitk(int dtype, int tile, const GemmArgs& a, hipStream_t stream) {
   if (tile == 128) {
     return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 2>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 2>(a, stream);
+  }
+  if (tile == 130) {  // 128 output features x 192 activation rows
+    return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 3>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 3>(a, stream);
   }
   if (tile == 129) {  // 128 output features x 256 activation rows
     return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 4>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 4>(a, stream);

@@ -93,7 +93,7 @@ def test_gateup_any_ff(capi, shape, dtype):
     assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "H %s" % (shape,))
 
 
-@pytest.mark.parametrize("variant", list(range(16)))
+@pytest.mark.parametrize("variant", list(range(17)))
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_every_tiled_variant(capi, variant, dtype):
     try:
@@ -218,7 +218,8 @@ def test_split_k_down_projection(capi, dtype):
     # the last three shapes are planned on 256 x 256 tiles (the last two with a K tail, the last with ragged M and d
     # as well), the others on 128 x 128 or 128 x 256
     for (M, d, ff) in [(200, 512, 4096), (130, 520, 2120), (65, 136, 8192), (256, 1024, 14336), (300, 264, 1032), (1024, 1024, 4096), (700, 2048, 2056), (768, 4096, 8192),
-                       (768, 4096, 8200), (1300, 3080, 8200)]:
+                       (768, 4096, 8200), (1300, 3080, 8200),
+                       (160, 4096, 4096), (250, 4096, 4104)]:  # one 128 x 192 / 128 x 256 tile of rows per workgroup
         inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=900 + M, x_scale=0.5)
         g = to_dev(inp)
         H = capi.gateup(g["X"], g["W13"])
