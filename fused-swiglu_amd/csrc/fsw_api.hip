@@ -60,7 +60,9 @@ int pick_tiled(int family, int64_t m, int64_t np) {
     // 10.5 us for 88 tiles of 128 x 128).
     // Up to 192 rows the tile is 128 x 192: the single-tile kernels are bound by their MFMA and LDS work as much as
     // by the weight stream (4096 x 28672, M = 160: 65 -> 54 us; 5120 x 27648: 89 -> 68 us).
-    if (family == 0 && m > 128 && m <= 256 && (np + 127) / 128 >= 128) return m <= 192 ? 16 : 15;
+    // 193 .. 256 rows: 128 x 256 on 8 waves, two per SIMD (4096 x 28672: 72 -> 64 us, 5120 x 27648: 94 -> 79-87 us
+    // against the 4-wave instance, variant 15).
+    if (family == 0 && m > 128 && m <= 256 && (np + 127) / 128 >= 128) return m <= 192 ? 16 : 17;
     return 7;
   }
   if (family == 0 && tiles256 > 256 && tiles256 <= 512) {

@@ -1157,6 +1157,7 @@ const TiledVariant kVariants[] = {
     {"ring5_256x192", 256, 192, 256},  // 192 activation rows: within 5 % of the default either way, not dispatched
     {"dma_128x256", 128, 256, 256},    // 129 .. 256 activation rows in ONE tile: every weight byte is read once
     {"dma_128x192", 128, 192, 256},    // the same for 129 .. 192 rows
+    {"dma8w_128x256", 128, 256, 512},  // 128 x 256 on 8 waves (two per SIMD), wave tile 64 x 64
 };
 
 int g_raster_group = 0;  // 0 = per-launch default
@@ -1184,11 +1185,11 @@ hipError_t launch_one(const GemmArgs& a, hipStream_t stream) {
 // of activation rows share them
 template <class E, bool GATED, bool KTAIL, int WP, int WQ, int FP, int FQ>
 void launch_dma_kernel(const dim3 grid, hipStream_t stream, const GemmArgs& a, int tiles_p, int tiles_q, int group) {
-  if constexpr (WP == 2 && WQ == 2 && FP == 2 && FQ >= 2 && FQ <= 4) {  // 128 weight rows x 128 / 192 / 256 activation rows
+  if constexpr (WP == 2 && FP == 2 && ((WQ == 2 && FQ >= 2 && FQ <= 4) || (WQ == 4 && FQ == 2))) {  // 128 weight rows x 128 / 192 / 256 activation rows
     // a single tile of activation rows: three stages (see NS). They leave room for one workgroup per compute unit,
     // so 128 x 128 launches of more than 256 workgroups keep two stages and two workgroups (8192 x 57344 at 65 rows,
     // 448 workgroups: 168 -> 158 us)
-    if (tiles_q == 1 && (FQ >= 3 || (long long)grid.x * grid.y <= 256)) {
+    if (tiles_q == 1 && (WQ * FQ >= 6 || (long long)grid.x * grid.y <= 256)) {
       hipLaunchKernelGGL((tiled_dma_kernel<E, GATED, KTAIL, WP, WQ, FP, FQ, true, 3>), grid, dim3(WP * WQ * 64), 0, stream,
                          a, tiles_p, tiles_q, group);
       return;
@@ -1311,6 +1312,7 @@ hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
     case 14: return launch_ring<E, GATED, 5, 2, 2, 4, 3>(a, stream);
     case 15: return launch_dma<E, GATED, 2, 2, 2, 4>(a, stream);
     case 16: return launch_dma<E, GATED, 2, 2, 2, 3>(a, stream);
+    case 17: return launch_dma<E, GATED, 2, 4, 2, 2>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -1446,8 +1448,8 @@ hipError_t launch_tiled_splitk(int dtype, int tile, const GemmArgs& a, hipStream
   if (tile == 130) {  // 128 output features x 192 activation rows
     return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 3>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 3>(a, stream);
   }
-  if (tile == 129) {  // 128 output features x 256 activation rows
-    return dtype == 0 ? launch_splitk_one<Bf16, 2, 2, 2, 4>(a, stream) : launch_splitk_one<Fp16, 2, 2, 2, 4>(a, stream);
+  if (tile == 129) {  // 128 output features x 256 activation rows, 8 waves
+    return dtype == 0 ? launch_splitk_one<Bf16, 2, 4, 2, 2>(a, stream) : launch_splitk_one<Fp16, 2, 4, 2, 2>(a, stream);
   }
   if (g_pair_ring == 2 && a.splits > 1) {  // 256 x 256 on the 16x16x32 kernel
     const hipError_t e = launch_pair16_splitk(dtype, a, stream);

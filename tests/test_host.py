@@ -124,7 +124,7 @@ def test_variant_choice_by_regime(capi):
     ws = capi.lib().fsw_down_workspace_bytes
     assert ws(0, 256, 4096, 14336) == 8 * 256 * 4096 * 4 and name(1, 256, 4096, 14336) == "splitk_dma_128x256"
     assert name(1, 160, 4096, 14336) == "splitk_dma_128x192" and name(0, 160, 28672, 4096) == "dma_128x192"
-    assert name(0, 256, 28672, 4096) == "dma_128x256"
+    assert name(0, 256, 28672, 4096) == "dma8w_128x256"
     assert name(1, 128, 4096, 14336) == "splitk_dma_128x128" and ws(0, 128, 4096, 14336) == 8 * 128 * 4096 * 4
     # above 256 rows: as many splits as keep all workgroups resident at once, on the tile the time estimate favours
     assert name(1, 257, 4096, 14336) == "splitk_dma_128x128" and ws(0, 257, 4096, 14336) == 5 * 257 * 4096 * 4

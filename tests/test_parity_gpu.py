@@ -93,7 +93,7 @@ def test_gateup_any_ff(capi, shape, dtype):
     assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "H %s" % (shape,))
 
 
-@pytest.mark.parametrize("variant", list(range(17)))
+@pytest.mark.parametrize("variant", list(range(18)))
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_every_tiled_variant(capi, variant, dtype):
     try:
