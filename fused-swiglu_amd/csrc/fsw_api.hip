@@ -77,12 +77,29 @@ int pick_tiled(int family, int64_t m, int64_t np) {
   return family == 0 ? 8 : 5;
 }
 
-int resolve_variant(int family, int64_t m, int64_t np) {
+// Most activation rows that still run the weight-streaming kernels (which take up to 64). Their time grows with
+// the rows (each workgroup re-reads every activation row from the L2), the tiled kernels' hardly does, and the
+// larger the weight matrices the earlier the tiled kernels win. Whole forwards, weight-streaming vs tiled, us:
+// 2048 x 8192: M = 32 32.5 / 37.1, 48 39.4 / 39.7, 64 46.0 / 41.7; 4096 x 11008: M = 32 57.7 / 60.4, 40 65.5 / 62.7,
+// 64 77.6 / 64.9; 4096 x 14336: M = 24 72.5 / 75.2, 32 75.3 / 70.4, 64 99.6 / 70.6; 8192 x 28672: M = 17 252.8 /
+// 228.3, 64 370.5 / 242.5. K == 0 stays with the weight-streaming kernels, which write the all-zero result.
+int64_t decode_rows(int family, int64_t np, int64_t k) {
+  if (k <= 0) return 64;
+  const int64_t d_ff = family == 0 ? (np / 2) * k : np * k;
+  return d_ff < ((int64_t)1 << 25) ? 48 : d_ff < ((int64_t)1 << 27) ? 32 : 16;
+}
+
+int resolve_variant(int family, int64_t m, int64_t np, int64_t k) {
   const int forced = g_forced_variant[family];
   if (forced == VARIANT_DECODE_FUSED || forced == VARIANT_DECODE_STREAM) return m <= 64 ? VARIANT_SKINNY : pick_tiled(family, m, np);
   if (forced >= 0 && !(forced == VARIANT_SKINNY && m > 64)) return forced;
-  if (m <= 64) return VARIANT_SKINNY;  // decode and small batches: weight streaming, HBM bound
+  if (m <= decode_rows(family, np, k)) return VARIANT_SKINNY;  // decode and small batches: weight streaming, HBM bound
   return pick_tiled(family, m, np);
+}
+
+// the weight-streaming kernels need no scratch and no blocked operands
+bool streams_weights(int family, int64_t m, int64_t np, int64_t k) {
+  return m <= 64 && resolve_variant(family, m, np, k) == VARIANT_SKINNY;
 }
 
 // M <= 16 with very large weight matrices runs on the persistent streaming kernel of kernels_decode.hip (one phase
@@ -151,7 +168,7 @@ static bool down_reblock_wanted(int64_t M, int64_t D, int64_t FF);
 const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, int64_t K_or_FF) {
   (void)dtype;
   if (family < 0 || family > 1) return "invalid";
-  const int v = resolve_variant(family, M, N_or_D);
+  const int v = resolve_variant(family, M, N_or_D, K_or_FF);
   if (v == VARIANT_SKINNY) return decode_stream_wanted(family, M, N_or_D, K_or_FF) ? "decode_stream" : "skinny";
   if (family == 1 && g_forced_variant[1] < 0 && M <= MAX_DIM && N_or_D > 0 && N_or_D <= MAX_DIM && K_or_FF > 0 &&
       K_or_FF <= MAX_DIM) {
@@ -216,7 +233,7 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
   a.np = (int)N;
   a.nq = (int)M;
   a.k = (int)K;
-  const int v = resolve_variant(0, M, N);
+  const int v = resolve_variant(0, M, N, K);
   if (v == VARIANT_SKINNY) {
     if (decode_stream_wanted(0, M, N, K)) {  // at most 16 rows: one 8-wave workgroup per CU, X held in registers
       fsw::DecodeArgs da = {};
@@ -244,14 +261,14 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
 // kernel on whole-line requests (8192 x 14336 x 4096: 0.10 ms of re-blocking + 0.62 ms against 0.80 ms for the
 // two-stage kernel on row-major H). Same rule for ragged panel counts as fsw_gateup_workspace_bytes.
 static bool down_reblock_wanted(int64_t M, int64_t D, int64_t FF) {
-  if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[1] >= 0 || pick_tiled(1, M, D) != 5) return false;
+  if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[1] >= 0 || pick_tiled(1, M, D) != 5) return false;  // 129 tiles or more
   if (M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM || fsw::tiled_split_plan((int)D, (int)M, (int)FF).splits > 1) return false;
   return M >= 1024 || M % 256 == 0;
 }
 
 size_t fsw_down_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
   (void)dtype;
-  if (M <= 64 || M > MAX_DIM || D <= 0 || D > MAX_DIM || FF <= 0 || FF > MAX_DIM) return 0;
+  if (M <= 0 || M > MAX_DIM || D <= 0 || D > MAX_DIM || FF <= 0 || FF > MAX_DIM || streams_weights(1, M, D, FF)) return 0;
   if (down_reblock_wanted(M, D, FF)) return (size_t)fsw::blocked_bytes(M, FF);
   const fsw::SplitPlan plan = fsw::tiled_split_plan((int)D, (int)M, (int)FF);
   return plan.splits > 1 ? (size_t)plan.splits * (size_t)M * (size_t)D * sizeof(float) : 0;
@@ -285,7 +302,7 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
   a.np = (int)D;
   a.nq = (int)M;
   a.k = (int)FF;
-  const int v = resolve_variant(1, M, D);
+  const int v = resolve_variant(1, M, D, FF);
   if (v == VARIANT_SKINNY) {
     if (decode_stream_wanted(1, M, D, FF)) {
       fsw::DecodeArgs da = {};
@@ -417,7 +434,7 @@ int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* Hb
 // kernel then reads whole cache lines: 1.52 -> 1.40 + 0.03 ms at 8192 x 4096 x 28672); H stays row-major.
 size_t fsw_gateup_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K) {
   (void)dtype;
-  if (M <= 64 || N <= 0 || K <= 0 || M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return 0;
+  if (M <= 64 || N <= 0 || K <= 0 || M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return 0;  // large tiles only
   if (g_forced_variant[0] >= 0 || pick_tiled(0, M, N) != 8) return 0;
   // Few activation panels with a ragged last one: the re-block launch and the zero rows of the padded panel (read
   // from memory, where the row-major kernel's out-of-range rows cost no traffic) outweigh the whole-line requests.
