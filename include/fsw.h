@@ -150,7 +150,8 @@ FSW_API int fsw_version(void);
 
 /*
  * Kernel-selection override for tuning and tests. family: 0 = gate/up, 1 = down; variant < 0 restores the
- * automatic choice by shape; variant 100 is the weight-streaming kernel (honoured for M <= 64); variant 102 is the
+ * automatic choice by shape; variant 100 is the weight-streaming kernel (honoured for M <= 64; the
+ * dispatcher itself picks it up to 16 .. 48 rows, the larger the weights the fewer); variant 102 is the
  * persistent streaming kernel (honoured for M <= 16; automatic only for d * ff >= 2^27); family 0 variant 101
  * makes fsw_mlp run M <= 16 as one persistent launch (gate/up, device-wide barrier, down) instead of two launches.
  * family 2 sets the raster band height of the tiled kernels instead (0 = per-kernel default).
