@@ -63,7 +63,8 @@ int pick_tiled(int family, int64_t m, int64_t np) {
     // 193 .. 256 rows: 128 x 256 on 8 waves, two per SIMD (4096 x 28672: 72 -> 64 us, 5120 x 27648: 94 -> 79-87 us
     // against the 4-wave instance, variant 15).
     if (family == 0 && m > 128 && m <= 256 && (np + 127) / 128 >= 128) return m <= 192 ? 16 : 17;
-    return 7;
+    // up to 64 rows the gate/up tile is 128 x 64 (4096 x 28672, M = 48: 39.4 -> 37.2 us)
+    return (family == 0 && m <= 64) ? 18 : 7;
   }
   if (family == 0 && tiles256 > 256 && tiles256 <= 512) {
     // A few large tiles more than compute units: the second round is nearly empty, while 128 x 128 tiles (two per
@@ -93,7 +94,15 @@ int resolve_variant(int family, int64_t m, int64_t np, int64_t k) {
   const int forced = g_forced_variant[family];
   if (forced == VARIANT_DECODE_FUSED || forced == VARIANT_DECODE_STREAM) return m <= 64 ? VARIANT_SKINNY : pick_tiled(family, m, np);
   if (forced >= 0 && !(forced == VARIANT_SKINNY && m > 64)) return forced;
-  if (m <= decode_rows(family, np, k)) return VARIANT_SKINNY;  // decode and small batches: weight streaming, HBM bound
+  if (m <= decode_rows(family, np, k)) {  // decode and small batches: weight streaming, HBM bound
+    // The gate/up product streams its weights faster through the three-stage 128 x 64 tiled kernel (direct-to-LDS
+    // copies) than through the weight-streaming kernel when its tiles of 128 weight rows fill one round of compute
+    // units and there are a dozen rows or more (gate/up, us: 4096 x 28672: M = 16 37.9 -> 35.6, 32 43.3 -> 36.0, M = 1
+    // level; 5120 x 27648: M = 16 49.3 -> 47.3, M = 4 45.3 -> 47.2; 172 tiles of 4096 x 22016: 28.8 -> 33.7, no).
+    const int64_t tiles = (np + 127) / 128;
+    if (family == 0 && m >= 12 && k > 0 && tiles >= 200 && tiles <= 256) return 18;
+    return VARIANT_SKINNY;
+  }
   return pick_tiled(family, m, np);
 }
 

@@ -1158,6 +1158,7 @@ const TiledVariant kVariants[] = {
     {"dma_128x256", 128, 256, 256},    // 129 .. 256 activation rows in ONE tile: every weight byte is read once
     {"dma_128x192", 128, 192, 256},    // the same for 129 .. 192 rows
     {"dma8w_128x256", 128, 256, 512},  // 128 x 256 on 8 waves (two per SIMD), wave tile 64 x 64
+    {"dma_128x64", 128, 64, 256},      // up to 64 activation rows in one tile
 };
 
 int g_raster_group = 0;  // 0 = per-launch default
@@ -1185,7 +1186,7 @@ hipError_t launch_one(const GemmArgs& a, hipStream_t stream) {
 // of activation rows share them
 template <class E, bool GATED, bool KTAIL, int WP, int WQ, int FP, int FQ>
 void launch_dma_kernel(const dim3 grid, hipStream_t stream, const GemmArgs& a, int tiles_p, int tiles_q, int group) {
-  if constexpr (WP == 2 && FP == 2 && ((WQ == 2 && FQ >= 2 && FQ <= 4) || (WQ == 4 && FQ == 2))) {  // 128 weight rows x 128 / 192 / 256 activation rows
+  if constexpr (WP == 2 && FP == 2 && ((WQ == 2 && FQ >= 1 && FQ <= 4) || (WQ == 4 && FQ == 2))) {  // 128 weight rows x 128 / 192 / 256 activation rows
     // a single tile of activation rows: three stages (see NS). They leave room for one workgroup per compute unit,
     // so 128 x 128 launches of more than 256 workgroups keep two stages and two workgroups (8192 x 57344 at 65 rows,
     // 448 workgroups: 168 -> 158 us)
@@ -1313,6 +1314,7 @@ hipError_t launch_variant(int variant, const GemmArgs& a, hipStream_t stream) {
     case 15: return launch_dma<E, GATED, 2, 2, 2, 4>(a, stream);
     case 16: return launch_dma<E, GATED, 2, 2, 2, 3>(a, stream);
     case 17: return launch_dma<E, GATED, 2, 4, 2, 2>(a, stream);
+    case 18: return launch_dma<E, GATED, 2, 2, 2, 1>(a, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -56,6 +56,12 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise FileNotFoundError(
                 "%s is missing: build it with `python setup.py build_hip` in %s" % (LIB_PATH, HERE))
+        # torch ships its own HIP runtime: when it is installed, load it first, so that this process holds one
+        # runtime only (loaded the other way round, the library's launches fail with FSW_E_DEVICE)
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in PROTOTYPES.items():
             fn = getattr(L, name)

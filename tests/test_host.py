@@ -105,16 +105,18 @@ def test_variant_choice_by_regime(capi):
     assert name(1, 8192, 4096, 14336) == "pair16_256x256"
     assert "256x256" in name(0, 4096, 22016, 4096)
     assert name(0, 512, 5632, 1024) == "dma_128x128"     # small problem: more, smaller tiles
-    assert name(0, 16, 28672, 4096) == "skinny" and name(1, 1, 4096, 14336) == "skinny"
+    assert name(0, 8, 28672, 4096) == "skinny" and name(1, 1, 4096, 14336) == "skinny"
     # the weight-streaming kernels take fewer rows the larger the weights: up to 48 / 32 / 16 rows
-    assert name(0, 32, 28672, 4096) == "skinny" and name(1, 32, 4096, 14336) == "skinny"
-    assert name(0, 33, 28672, 4096) == "dma_128x128" and name(1, 33, 4096, 14336) == "splitk_dma_128x128"
-    assert name(0, 48, 2 * 8192, 2048) == "skinny" and name(0, 49, 2 * 8192, 2048) == "dma_128x128"
+    assert name(0, 32, 22016, 4096) == "skinny" and name(1, 32, 4096, 14336) == "skinny"
+    assert name(0, 33, 28672, 4096) == "dma_128x64" and name(1, 33, 4096, 14336) == "splitk_dma_128x128"
+    assert name(0, 48, 2 * 8192, 2048) == "skinny" and name(0, 49, 2 * 8192, 2048) == "dma_128x64"
+    # gate/up with 200 .. 256 tiles of 128 weight rows and a dozen rows or more: the 128 x 64 tiled kernel streams faster
+    assert name(0, 16, 28672, 4096) == "dma_128x64" and name(0, 11, 28672, 4096) == "skinny"
     assert name(0, 64, 28672, 0) == "skinny"
     assert name(0, 100, 28672, 4096) == "dma_128x128"
     # at most 16 rows and d * ff >= 2^27: the persistent streaming kernel, one projection per launch
     assert name(0, 16, 2 * 28672, 8192) == "decode_stream" and name(1, 16, 8192, 28672) == "decode_stream"
-    assert name(0, 17, 2 * 28672, 8192) == "dma_128x128"
+    assert name(0, 17, 2 * 28672, 8192) == "dma_128x64"
     L = capi.lib()
     try:
         assert L.fsw_set_variant(0, 102) == capi.OK and L.fsw_set_variant(1, 100) == capi.OK

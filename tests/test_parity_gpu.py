@@ -93,7 +93,7 @@ def test_gateup_any_ff(capi, shape, dtype):
     assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "H %s" % (shape,))
 
 
-@pytest.mark.parametrize("variant", list(range(18)))
+@pytest.mark.parametrize("variant", list(range(19)))
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_every_tiled_variant(capi, variant, dtype):
     try:
@@ -169,7 +169,7 @@ def test_streaming_decode_variant(capi, M, dtype):
         capi.set_variant(0, -1)
         capi.set_variant(1, -1)
     assert capi.variant_name(0, 0, 16, 2 * 28672, 8192) == "decode_stream"
-    assert capi.variant_name(0, 0, 16, 2 * 14336, 4096) == "skinny"
+    assert capi.variant_name(0, 0, 16, 2 * 14336, 4096) == "dma_128x64" and capi.variant_name(1, 0, 16, 4096, 14336) == "skinny"
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
