@@ -29,9 +29,9 @@ sys.path.insert(0, os.path.join(ROOT, "fused-swiglu_amd"))
 MFMA_PEAK_TFLOPS = 2516.6  # MI355X dense bf16/fp16: 256 CU x 2.4 GHz x 4096 flop/clk/CU
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 # L2<->fabric bytes per launch of the dominant kernel, from separate `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
-# runs scaled by a 1 GiB copy kernel (profiles/tiled_prefill_C3_hbm_traffic_pmc.md, skinny_decode_C4_kernel_trace.md);
+# runs scaled by a 1 GiB copy kernel (profiles/tiled_prefill_C3_hbm_traffic_pmc.md, decode_C4_kernel_trace.md);
 # not measurable in-process. C3: the gate/up kernel; C4: both decode kernels together.
-MEASURED_TRAFFIC_BYTES = {"C3": 2753094 * 1024 + 229376 * 1024, "C4": (230454 + 118324 + 448 + 128) * 1024}
+MEASURED_TRAFFIC_BYTES = {"C3": 2753094 * 1024 + 229376 * 1024, "C4": (231450 + 118322 + 448 + 128) * 1024}
 
 
 DECODE_WARMUP = 500  # untimed forwards before the HBM-bound (M = 16) measurement, ~30 ms
