@@ -4,17 +4,22 @@
 #include <hip/hip_runtime.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "fsw.h"
 #include "fsw_internal.h"
 
 namespace {
 
 thread_local int g_last_hip_error = 0;
-int g_forced_variant[2] = {-1, -1};  // family 0 = gate/up, 1 = down
+// Kernel override of fsw_set_variant, per calling thread: a thread's workspace queries and launches always agree,
+// and no thread can change another's kernel choice. family 0 = gate/up, 1 = down.
+thread_local int g_forced_variant[2] = {-1, -1};
 
 constexpr int VARIANT_SKINNY = 100;          // id of the weight-streaming kernel in fsw_set_variant
 constexpr int VARIANT_DECODE_STREAM = 102;   // M <= 16: the streaming kernel of kernels_decode.hip, one phase per launch
 constexpr int VARIANT_DECODE_FUSED = 101;    // fsw_mlp only: single-launch decode forward (family 0)
+constexpr int VARIANT_DECODE_FUSED_FAIL = 103;  // 101 with a device-wide barrier that cannot complete (failure-path test)
 constexpr int64_t MAX_DIM = 1LL << 30;       // every size is cast to int inside the kernels
 constexpr int64_t MAX_LD = 1LL << 21;        // keeps tile-relative byte offsets below 2^31
 
@@ -22,7 +27,7 @@ bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
 // gfx950 check, cached per device ordinal.
 int check_device() {
-  static int ok_mask[64] = {0};  // 0 unknown, 1 ok, 2 not gfx950
+  static std::atomic<int> ok_mask[64];  // 0 unknown, 1 ok, 2 not gfx950 (zero-initialised; racing writers agree)
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) {
@@ -30,17 +35,22 @@ int check_device() {
     return FSW_E_DEVICE;
   }
   if (dev < 0 || dev >= 64) return FSW_E_DEVICE;
-  if (ok_mask[dev] == 0) {
+  int state = ok_mask[dev].load(std::memory_order_relaxed);
+  if (state == 0) {
     hipDeviceProp_t prop;
     e = hipGetDeviceProperties(&prop, dev);
     if (e != hipSuccess) {
       g_last_hip_error = (int)e;
       return FSW_E_DEVICE;
     }
-    ok_mask[dev] = (strncmp(prop.gcnArchName, "gfx950", 6) == 0) ? 1 : 2;
+    state = (strncmp(prop.gcnArchName, "gfx950", 6) == 0) ? 1 : 2;
+    ok_mask[dev].store(state, std::memory_order_relaxed);
   }
-  return ok_mask[dev] == 1 ? FSW_OK : FSW_E_DEVICE;
+  return state == 1 ? FSW_OK : FSW_E_DEVICE;
 }
+
+// indices of the tiled kernels (tiled_variant() of kernels_tiled.hip)
+constexpr int V_128x128 = 0, V_128x192 = 2, V_8W_128x256 = 3, V_128x64 = 4, V_256x256 = 5;
 
 // Variant choice for the tiled kernels: the widest tile whose activation-row extent is not mostly padding,
 // stepping down to 128x128 when a 256-wide grid would leave most of the 256 CUs idle.
@@ -62,9 +72,9 @@ int pick_tiled(int family, int64_t m, int64_t np) {
     // by the weight stream (4096 x 28672, M = 160: 65 -> 54 us; 5120 x 27648: 89 -> 68 us).
     // 193 .. 256 rows: 128 x 256 on 8 waves, two per SIMD (4096 x 28672: 72 -> 64 us, 5120 x 27648: 94 -> 79-87 us
     // against the 4-wave instance, variant 15).
-    if (family == 0 && m > 128 && m <= 256 && (np + 127) / 128 >= 128) return m <= 192 ? 16 : 17;
+    if (family == 0 && m > 128 && m <= 256 && (np + 127) / 128 >= 128) return m <= 192 ? V_128x192 : V_8W_128x256;
     // up to 64 rows the gate/up tile is 128 x 64 (4096 x 28672, M = 48: 39.4 -> 37.2 us)
-    return (family == 0 && m <= 64) ? 18 : 7;
+    return (family == 0 && m <= 64) ? V_128x64 : V_128x128;
   }
   if (family == 0 && tiles256 > 256 && tiles256 <= 512) {
     // A few large tiles more than compute units: the second round is nearly empty, while 128 x 128 tiles (two per
@@ -72,10 +82,9 @@ int pick_tiled(int family, int64_t m, int64_t np) {
     // workgroups: ~33 us against ~75-100 us at K = 4096; the small tile must win by 20 % to be taken. 4096 x 36864,
     // M = 300 (288 tiles): 151 -> 130 us; 4096 x 22016, M = 640 (258 tiles): 148 -> 119 us.
     const int64_t tiles128 = ((np + 127) / 128) * ((m + 127) / 128);
-    if (((tiles128 + 255) / 256) * 44 < ((tiles256 + 255) / 256) * 100) return 7;
+    if (((tiles128 + 255) / 256) * 44 < ((tiles256 + 255) / 256) * 100) return V_128x128;
   }
-  // 256 x 256: the gate/up product runs best on the four-stage ring, the deep-K down product on two stages
-  return family == 0 ? 8 : 5;
+  return V_256x256;
 }
 
 // Most activation rows that still run the weight-streaming kernels (which take up to 64). Their time grows with
@@ -92,7 +101,8 @@ int64_t decode_rows(int family, int64_t np, int64_t k) {
 
 int resolve_variant(int family, int64_t m, int64_t np, int64_t k) {
   const int forced = g_forced_variant[family];
-  if (forced == VARIANT_DECODE_FUSED || forced == VARIANT_DECODE_STREAM) return m <= 64 ? VARIANT_SKINNY : pick_tiled(family, m, np);
+  if (forced == VARIANT_DECODE_FUSED || forced == VARIANT_DECODE_FUSED_FAIL || forced == VARIANT_DECODE_STREAM)
+    return m <= 64 ? VARIANT_SKINNY : pick_tiled(family, m, np);
   if (forced >= 0 && !(forced == VARIANT_SKINNY && m > 64)) return forced;
   if (m <= decode_rows(family, np, k)) {  // decode and small batches: weight streaming, HBM bound
     // The gate/up product streams its weights faster through the three-stage 128 x 64 tiled kernel (direct-to-LDS
@@ -100,7 +110,7 @@ int resolve_variant(int family, int64_t m, int64_t np, int64_t k) {
     // units and there are a dozen rows or more (gate/up, us: 4096 x 28672: M = 16 37.9 -> 35.6, 32 43.3 -> 36.0, M = 1
     // level; 5120 x 27648: M = 16 49.3 -> 47.3, M = 4 45.3 -> 47.2; 172 tiles of 4096 x 22016: 28.8 -> 33.7, no).
     const int64_t tiles = (np + 127) / 128;
-    if (family == 0 && m >= 12 && k > 0 && tiles >= 200 && tiles <= 256) return 18;
+    if (family == 0 && m >= 12 && k > 0 && tiles >= 200 && tiles <= 256) return V_128x64;
     return VARIANT_SKINNY;
   }
   return pick_tiled(family, m, np);
@@ -154,18 +164,18 @@ const char* fsw_strerror(int code) {
 
 int fsw_last_hip_error(void) { return g_last_hip_error; }
 
+int fsw_decode_barrier_failures(void) {
+  const int drc = check_device();
+  if (drc != FSW_OK) return drc;
+  int count = 0;
+  const int rc = finish(fsw::decode_barrier_failures(&count));
+  return rc != FSW_OK ? rc : count;
+}
+
 int fsw_set_variant(int family, int variant) {
-  if (family == 2) {  // tuning knob: raster band height of the tiled kernels
-    fsw::set_raster_group(variant);
-    return FSW_OK;
-  }
-  if (family == 3) {  // tuning knob: kernel behind the blocked entry points when the weights are row-major
-    fsw::set_pair_ring(variant);
-    return FSW_OK;
-  }
   if (family < 0 || family > 1) return FSW_E_VARIANT;
   if (variant >= 0 && variant != VARIANT_SKINNY && variant != VARIANT_DECODE_STREAM &&
-      !(family == 0 && variant == VARIANT_DECODE_FUSED) &&
+      !(family == 0 && (variant == VARIANT_DECODE_FUSED || variant == VARIANT_DECODE_FUSED_FAIL)) &&
       variant >= fsw::tiled_variant_count())
     return FSW_E_VARIANT;
   g_forced_variant[family] = variant < 0 ? -1 : variant;
@@ -186,10 +196,9 @@ const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, i
       if (plan.tile == 128) return "splitk_dma_128x128";
       if (plan.tile == 129) return "splitk_dma_128x256";
       if (plan.tile == 130) return "splitk_dma_128x192";
-      return fsw::pair_ring_mode() == 2 ? "splitk_pair16_256x256" : "splitk_dma_256x256";
+      return "splitk_pair16_256x256";
     }
   }
-  if ((v == 8 || v == 5) && g_forced_variant[family] < 0 && fsw::pair_ring_mode() == 2) return "pair16_256x256";
   return fsw::tiled_variant(v).name;
 }
 
@@ -259,10 +268,6 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
     }
     return finish(fsw::launch_skinny(dtype, true, a, nullptr, (hipStream_t)stream));
   }
-  if (v == 8 && g_forced_variant[0] < 0 && fsw::pair_ring_mode() == 2) {
-    a.layout = 0;  // 256 x 256 tiles on row-major operands: the 16x16x32 pair ring with row-major activations
-    return finish(fsw::launch_tiled_blocked(dtype, true, a, (hipStream_t)stream));
-  }
   return finish(fsw::launch_tiled(v, dtype, true, a, (hipStream_t)stream));
 }
 
@@ -270,7 +275,7 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
 // kernel on whole-line requests (8192 x 14336 x 4096: 0.10 ms of re-blocking + 0.62 ms against 0.80 ms for the
 // two-stage kernel on row-major H). Same rule for ragged panel counts as fsw_gateup_workspace_bytes.
 static bool down_reblock_wanted(int64_t M, int64_t D, int64_t FF) {
-  if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[1] >= 0 || pick_tiled(1, M, D) != 5) return false;  // 129 tiles or more
+  if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[1] >= 0 || pick_tiled(1, M, D) != V_256x256) return false;  // 129 tiles or more
   if (M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM || fsw::tiled_split_plan((int)D, (int)M, (int)FF).splits > 1) return false;
   return M >= 1024 || M % 256 == 0;
 }
@@ -279,6 +284,7 @@ size_t fsw_down_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
   (void)dtype;
   if (M <= 0 || M > MAX_DIM || D <= 0 || D > MAX_DIM || FF <= 0 || FF > MAX_DIM || streams_weights(1, M, D, FF)) return 0;
   if (down_reblock_wanted(M, D, FF)) return (size_t)fsw::blocked_bytes(M, FF);
+  if (g_forced_variant[1] >= 0) return 0;  // a forced kernel runs unsplit
   const fsw::SplitPlan plan = fsw::tiled_split_plan((int)D, (int)M, (int)FF);
   return plan.splits > 1 ? (size_t)plan.splits * (size_t)M * (size_t)D * sizeof(float) : 0;
 }
@@ -335,10 +341,6 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
     a.partial = (float*)workspace;
     return finish(fsw::launch_tiled_splitk(dtype, plan.tile, a, (hipStream_t)stream));
   }
-  if (v == 5 && g_forced_variant[1] < 0 && fsw::pair_ring_mode() == 2) {
-    a.layout = 0;
-    return finish(fsw::launch_tiled_blocked(dtype, false, a, (hipStream_t)stream));
-  }
   return finish(fsw::launch_tiled(v, dtype, false, a, (hipStream_t)stream));
 }
 
@@ -347,7 +349,7 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
 static bool blocked_regime(int64_t M, int64_t D, int64_t FF) {
   if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[0] >= 0 || g_forced_variant[1] >= 0) return false;
   if (M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM / 2) return false;
-  return pick_tiled(0, M, 2 * FF) == 8 && pick_tiled(1, M, D) == 5 &&
+  return pick_tiled(0, M, 2 * FF) == V_256x256 && pick_tiled(1, M, D) == V_256x256 &&
          fsw::tiled_split_plan((int)D, (int)M, (int)FF).splits == 1;  // a split-K down projection reads row-major H
 }
 
@@ -409,7 +411,7 @@ int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* X
   a.nq = (int)M;
   a.k = (int)K;
   a.layout = 1 | (ldh == 0 ? 2 : 0) | (w_blocked ? 4 : 0);
-  return finish(fsw::launch_tiled_blocked(dtype, true, a, (hipStream_t)stream));
+  return finish(fsw::launch_pair16(dtype, true, a, (hipStream_t)stream));
 }
 
 int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* Hb, const void* W2, int64_t ldw2,
@@ -436,7 +438,7 @@ int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* Hb
   a.nq = (int)M;
   a.k = (int)FF;
   a.layout = w_blocked ? 5 : 1;
-  return finish(fsw::launch_tiled_blocked(dtype, false, a, (hipStream_t)stream));
+  return finish(fsw::launch_pair16(dtype, false, a, (hipStream_t)stream));
 }
 
 // fsw_gateup with caller scratch: in the large-tile regime X is re-blocked into the scratch first (the gated
@@ -444,7 +446,7 @@ int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* Hb
 size_t fsw_gateup_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K) {
   (void)dtype;
   if (M <= 64 || N <= 0 || K <= 0 || M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return 0;  // large tiles only
-  if (g_forced_variant[0] >= 0 || pick_tiled(0, M, N) != 8) return 0;
+  if (g_forced_variant[0] >= 0 || pick_tiled(0, M, N) != V_256x256) return 0;
   // Few activation panels with a ragged last one: the re-block launch and the zero rows of the padded panel (read
   // from memory, where the row-major kernel's out-of-range rows cost no traffic) outweigh the whole-line requests.
   // Measured at 4096 x 28672, blocked vs row-major ring: M = 384: 145 vs 129 us, 576: 215 vs 190, 640: 216 vs 199,
@@ -479,10 +481,14 @@ size_t fsw_mlp_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
          fsw_gateup_workspace_bytes(dtype, M, 2 * FF, D);
 }
 
-int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t ldx, const void* W13, int64_t ldw13,
-            const void* W2, int64_t ldw2, void* Y, int64_t ldy, void* workspace, size_t workspace_bytes,
-            void* stream) {
-  if (M < 0 || D < 0 || FF < 0 || FF > MAX_DIM / 2) return FSW_E_SHAPE;
+// single_launch_ok: whether the opt-in single-launch decode forward may be used (it creates events on first use,
+// which the entry point that must not allocate cannot afford)
+static int mlp_impl(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t ldx, const void* W13,
+                    int64_t ldw13, const void* W2, int64_t ldw2, void* Y, int64_t ldy, void* workspace,
+                    size_t workspace_bytes, void* stream, bool single_launch_ok) {
+  if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
+  if (M < 0 || D < 0 || FF < 0 || M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM / 2) return FSW_E_SHAPE;
+  if (M == 0 || D == 0) return FSW_OK;  // Y is empty: nothing to read or write
   const size_t need = fsw_mlp_workspace_bytes(dtype, M, D, FF);
   if (need > 0 && (!workspace || workspace_bytes < need)) return FSW_E_WORKSPACE;
   if (need > 0 && !aligned16(workspace)) return FSW_E_ALIGN;
@@ -493,10 +499,11 @@ int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t 
   if (rc != FSW_OK) return rc;
   rc = fsw_validate_down(dtype, M, D, FF, Hbuf, FF, W2, ldw2, Y, ldy);
   if (rc != FSW_OK) return rc;
-  if (M == 0 || D == 0) return FSW_OK;
-  if (M <= 16 && FF > 0 && g_forced_variant[0] == VARIANT_DECODE_FUSED) {
+  if (single_launch_ok && M <= 16 && FF > 0 &&
+      (g_forced_variant[0] == VARIANT_DECODE_FUSED || g_forced_variant[0] == VARIANT_DECODE_FUSED_FAIL)) {
     // opt-in: one persistent launch does both projections with a device-wide barrier in between. Measured
     // slower than the two weight-streaming launches so far (stragglers before the barrier), so not the default.
+    // Without a free barrier slot, or on a stream that is being captured, it is the two launches below.
     fsw::DecodeArgs da;
     da.X = X;
     da.W13 = W13;
@@ -514,7 +521,10 @@ int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t 
     if (fsw::decode_mlp_supported(da, 3)) {
       const int drc = check_device();
       if (drc != FSW_OK) return drc;
-      return finish(fsw::launch_decode_mlp(dtype, da, (hipStream_t)stream));
+      bool launched = false;
+      const int lrc = finish(fsw::launch_decode_mlp(dtype, da, (hipStream_t)stream, 3, &launched,
+                                                    g_forced_variant[0] == VARIANT_DECODE_FUSED_FAIL));
+      if (lrc != FSW_OK || launched) return lrc;
     }
   }
   if (blocked_regime(M, D, FF)) {  // workspace = [H blocked][X blocked]
@@ -532,6 +542,12 @@ int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t 
                      fsw_gateup_workspace_bytes(dtype, M, 2 * FF, D), stream);
   if (rc != FSW_OK) return rc;
   return fsw_down(dtype, M, D, FF, Hbuf, FF, W2, ldw2, Y, ldy, ws2, down_ws, stream);
+}
+
+int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t ldx, const void* W13, int64_t ldw13,
+            const void* W2, int64_t ldw2, void* Y, int64_t ldy, void* workspace, size_t workspace_bytes,
+            void* stream) {
+  return mlp_impl(dtype, M, D, FF, X, ldx, W13, ldw13, W2, ldw2, Y, ldy, workspace, workspace_bytes, stream, true);
 }
 
 }  // extern "C"

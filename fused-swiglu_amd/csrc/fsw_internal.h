@@ -20,7 +20,7 @@ struct GemmArgs {
   // store fp32 partial sums to partial[split][nq][np]; splitk_reduce() sums them and rounds once.
   int splits = 1;
   float* partial = nullptr;
-  // panel-blocked operands / output of the 256 x 256 ring kernel (launch_tiled_blocked): bit 0 = Q, bit 1 = O
+  // panel-blocked operands / output of the 256 x 256 kernel (launch_pair16): bit 0 = Q, bit 1 = O
   // (gated kernel), bit 2 = P. A blocked [rows, k] matrix is ceil(rows / 256) panels of ceil(k / 32) blocks of
   // [256 rows][64 bytes], zero padded (blocked_bytes()).
   int layout = 0;
@@ -35,19 +35,17 @@ struct TiledVariant {
   int bp, bq;        // workgroup tile: weight rows x activation rows
   int threads;
 };
-void set_pair_ring(int on);    // blocked entry points with row-major weights: pair ring (default) or plain ring
-void set_raster_group(int g);  // activation-row tiles per raster band; 0 restores the per-kernel default
 int tiled_variant_count();
+int pair16_variant();  // index of the 256 x 256 kernel in the table
 const TiledVariant& tiled_variant(int variant);
+// row-major operands (GemmArgs::layout 0)
 hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
-// gated: X blocked in (bit 0), H blocked out (bit 1) or row-major, W13 blocked (bit 2) or row-major: layouts 1, 3, 5, 7;
-// plain: H blocked in, W2 row-major (1) or blocked (5)
 int raster_group(bool gated);  // activation-row tiles per raster band of the tiled kernels
-// the 16x16x32 pair-ring kernel (kernels_pair16.hip) for GemmArgs::layout 0, 1, 3, 5, 7
+// The 256 x 256 kernel on v_mfma_f32_16x16x32 (kernels_pair16.hip) for GemmArgs::layout 0, 1, 3, 5, 7.
+// gated: X blocked in (bit 0), H blocked out (bit 1) or row-major, W13 blocked (bit 2) or row-major: layouts 1, 3, 5, 7;
+// plain: H blocked in, W2 row-major (1) or blocked (5); 0 = everything row-major
 hipError_t launch_pair16(int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
 hipError_t launch_pair16_splitk(int dtype, const GemmArgs& a, hipStream_t stream);  // partials only, no reduction
-int pair_ring_mode();  // kernel family behind the 256 x 256 tiles: 2 = 16x16x32 pair ring, 1 / 0 = 32x32x16 kernels
-hipError_t launch_tiled_blocked(int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
 // row-major [rows, k] (row stride ld elements) -> blocked; gated_order: W13's up/gate rows de-interleaved per panel
 hipError_t launch_block_rows(const void* src, long long ld, int rows, int k, void* dst, bool gated_order,
                              hipStream_t stream);
@@ -85,7 +83,11 @@ struct DecodeArgs {
   int nq, d, ff;
 };
 bool decode_mlp_supported(const DecodeArgs& a, int phases = 3);
-// phases: 1 = gate/up only, 2 = down only (H already written), 3 = both in one launch
-hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream, int phases = 3);
+// phases: 1 = gate/up only, 2 = down only (H already written), 3 = both in one launch. With phases == 3 *launched
+// tells whether the launch was enqueued: it is not (and the call still succeeds) when no barrier slot is free or the
+// stream is being captured. test_unreachable makes the device-wide barrier give up at once (failure-path test).
+hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream, int phases, bool* launched = nullptr,
+                             bool test_unreachable = false);
+hipError_t decode_barrier_failures(int* count);
 
 }  // namespace fsw

@@ -27,9 +27,14 @@
 // this kernel reads H before the barrier), so the plain loads of phase 2 miss and fetch the written data.
 //
 // Device-wide barrier: arrive/depart counters in a file-scope __device__ array (zero at module load, restored to
-// zero by the last workgroup to depart); the host hands concurrent launches different slots. The spin is bounded:
-// if the workgroups are not all resident (someone else holds CUs) the kernel gives up, sets the slot's `failed`
-// word (left set, for diagnosis) and finishes instead of hanging.
+// zero by the last workgroup to depart). The host hands every single-launch forward a slot of its own and reuses a
+// slot only when the event recorded behind its previous launch has completed; with no free slot, or on a stream
+// that is being captured, the caller runs the two-launch path instead. The spin is bounded: if the workgroups are
+// not all resident (someone else holds CUs) a workgroup gives up, sets the slot's `failed` word and SKIPS the down
+// projection, as does every workgroup that sees the word set after the barrier: a failed launch leaves Y
+// incomplete and is reported by decode_barrier_failures(), it never hangs and never multiplies a partial H.
+#include <mutex>
+
 #include "fsw_internal.h"
 #include "fsw_device.h"
 
@@ -39,26 +44,25 @@ constexpr int DEC_NW = 8;            // waves per workgroup
 constexpr int DEC_XS = 4;            // phase 1: K steps whose activations a wave holds at once = weight steps in flight
 constexpr int DEC_TG = 8;            // phase 1: tiles (accumulators) per pass
 constexpr int DEC_PF2 = 4;           // phase 2: weight steps in flight per wave
-#ifndef DEC_POLL_SLEEP
-#define DEC_POLL_SLEEP 8
-#endif
-#ifndef DEC_FILL_LATE
-#define DEC_FILL_LATE 0
-#endif
-constexpr int DEC_SLOTS = 64;        // barrier slots for concurrent launches
+constexpr int DEC_POLL_SLEEP = 8;    // s_sleep between polls: 256 pollers must not saturate the counter's channel
+constexpr int DEC_SLOTS = 64;        // barrier slots for launches in flight at the same time
 constexpr unsigned DEC_SPIN_LIMIT = 1u << 18;  // ~0.3 s of polling
 static __device__ unsigned g_dec_barrier[DEC_SLOTS * 4];  // per slot: arrive, depart, failed, pad
 
-// phases: bit 0 = gate/up, bit 1 = down; 3 = both with the device-wide barrier in between
+// phases: bit 0 = gate/up, bit 1 = down; 3 = both with the device-wide barrier in between, which waits until
+// `expected` workgroups have arrived (the grid size; a test passes more, so that the bounded wait gives up) for at
+// most `spin_limit` polls.
 template <class E>
 __global__ void __launch_bounds__(DEC_NW * 64)
-decode_mlp_kernel(const DecodeArgs a, unsigned* bar, const int phases) {
+decode_mlp_kernel(const DecodeArgs a, unsigned* bar, const int phases, const unsigned expected,
+                  const unsigned spin_limit) {
   constexpr int KS = 128;
   // slabs of the waves first; the phase-1 reduction reuses everything, the phase-2 reduction has its own two
   // buffers behind the slabs
   constexpr int LDS_BYTES = (DEC_NW * DEC_TG * 1024 > 2 * DEC_NW * 4096 + 2 * DEC_NW * 1024) ? DEC_NW * DEC_TG * 1024
                                                                                             : 2 * DEC_NW * 4096 + 2 * DEC_NW * 1024;
   __shared__ __align__(16) unsigned char lds[LDS_BYTES];
+  __shared__ unsigned barrier_failed;  // single launch: set by thread 0 when the device-wide barrier did not complete
 
   const int t = threadIdx.x;
   const int lane = t & 63;
@@ -243,30 +247,33 @@ decode_mlp_kernel(const DecodeArgs a, unsigned* bar, const int phases) {
   // phase 1 early spends its wait fetching W2; a late one arrives without waiting for its own ring.
   u32x4 w2[DEC_PF2][4];
   if (phases == 3) {
-    __syncthreads();  // vmcnt(0): every store of H by this workgroup has been acknowledged by memory
+    // every store of H by this wave has been acknowledged by memory (written out: the fences of a workgroup
+    // barrier need not wait for vmcnt), then every wave of the workgroup has got here
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if (threadIdx.x == 0) __hip_atomic_fetch_add(bar + 0, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  // Wave 0 polls the barrier, and loads return in order: with its own ring fill in flight (queued behind every
-  // other workgroup's) the poll result would arrive microseconds late, so wave 0 fills its ring after the barrier.
-  auto fill_ring = [&]() {
+  if (phases & 2) {
 #pragma unroll
     for (int j = 0; j < DEC_PF2; ++j) {
       next_w(w2[j]);
       __builtin_amdgcn_sched_barrier(0);
     }
-  };
-  const bool fill_late = (phases == 3) && wave == 0 && DEC_FILL_LATE;
-  if ((phases & 2) && !fill_late) fill_ring();
+  }
+  bool skip_down = false;
   if (phases == 3) {
     if (threadIdx.x == 0) {
-      unsigned spins = 0;
-      while (__hip_atomic_load(bar + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gridDim.x) {
-        if (++spins > DEC_SPIN_LIMIT) {  // not all workgroups are resident: give up rather than hang
+      unsigned spins = 0, failed = 0;
+      while (__hip_atomic_load(bar + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < expected) {
+        if (++spins > spin_limit) {  // not all workgroups are resident: give up rather than hang
           __hip_atomic_store(bar + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          failed = 1;
           break;
         }
-        __builtin_amdgcn_s_sleep(DEC_POLL_SLEEP);  // 256 pollers must not saturate the counter's channel
+        __builtin_amdgcn_s_sleep(DEC_POLL_SLEEP);
       }
+      // a workgroup that got through still skips the down projection when another one has given up
+      if (!failed) failed = __hip_atomic_load(bar + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      barrier_failed = failed;
       // depart: the last workgroup out restores the slot for the next launch that is handed it
       const unsigned left = __hip_atomic_fetch_add(bar + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (left == gridDim.x - 1) {
@@ -275,11 +282,11 @@ decode_mlp_kernel(const DecodeArgs a, unsigned* bar, const int phases) {
       }
     }
     lds_barrier();  // no vmcnt wait: the ring stays in flight; also keeps loads of H below the barrier
-    if (fill_late) fill_ring();
+    skip_down = barrier_failed != 0;
   }
 
   // ---------------------------------------------------------------- phase 2: Y = H W2^T
-  if (phases & 2) {
+  if ((phases & 2) && !skip_down) {
     float* part_all = (float*)(lds + 2 * DEC_NW * 4096);  // two buffers of [wave][lane][4], by tile parity
     // H fragments ride the same ring distance as the weights and are issued before them: loads return in
     // order, so a younger, shorter H ring would make every step wait for the weight loads issued ahead of it
@@ -359,37 +366,116 @@ bool decode_mlp_supported(const DecodeArgs& a, int phases) {
   return true;
 }
 
-hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream, int phases) {
-  static int cu_count[64] = {0};
-  static unsigned* bar_base[64] = {nullptr};
-  static unsigned next_slot = 0;
-  if (phases < 1 || phases > 3) return hipErrorInvalidValue;
+namespace {
+
+// per-device barrier slots of the single-launch forward
+struct DecodeDevice {
+  int cu_count = 0;
+  unsigned* bar = nullptr;           // device address of g_dec_barrier on this device
+  hipEvent_t done[DEC_SLOTS] = {};   // recorded behind the last launch that used the slot
+  bool used[DEC_SLOTS] = {};
+  unsigned next = 0;
+};
+std::mutex g_dec_mutex;
+DecodeDevice g_dec_dev[64];
+
+// device ordinal and its state, initialised on first use (under g_dec_mutex)
+hipError_t decode_device(DecodeDevice*& out) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
-  if (cu_count[dev] == 0) {
+  DecodeDevice& d = g_dec_dev[dev];
+  if (d.cu_count == 0) {
     hipDeviceProp_t prop;
     e = hipGetDeviceProperties(&prop, dev);
     if (e != hipSuccess) return e;
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_dec_barrier));
     if (e != hipSuccess) return e;
-    bar_base[dev] = (unsigned*)p;
-    cu_count[dev] = prop.multiProcessorCount;
+    d.bar = (unsigned*)p;
+    d.cu_count = prop.multiProcessorCount;
   }
-  const unsigned slot = __atomic_fetch_add(&next_slot, 1u, __ATOMIC_RELAXED) % DEC_SLOTS;
-  unsigned* bar = bar_base[dev] + slot * 4;
+  out = &d;
+  return hipSuccess;
+}
+
+}  // namespace
+
+// phases 1 and 2 are plain launches. phases == 3 (one launch, device-wide barrier) needs a barrier slot that no
+// launch in flight is using: *launched is set to false, and nothing is enqueued, when there is none or when `stream`
+// is being captured (a replayed graph could run twice at once on one slot) -- the caller then runs two launches.
+// test_unreachable: the barrier waits for one arrival more than the grid has and polls 64 times only, so that
+// every workgroup takes the give-up path and the kernel still ends normally.
+hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream, int phases, bool* launched,
+                             bool test_unreachable) {
+  if (launched) *launched = false;
+  if (phases < 1 || phases > 3) return hipErrorInvalidValue;
+  std::lock_guard<std::mutex> lock(g_dec_mutex);
+  DecodeDevice* d = nullptr;
+  hipError_t e = decode_device(d);
+  if (e != hipSuccess) return e;
   const int tiles1 = (phases & 1) ? (2 * a.ff + 15) / 16 : 0, tiles2 = (phases & 2) ? (a.d + 15) / 16 : 0;
-  int grid = cu_count[dev];  // one workgroup per CU: all resident at once, which the barrier relies on
+  int grid = d->cu_count;  // one workgroup per CU: all resident at once, which the barrier relies on
   const int most = tiles1 > tiles2 ? tiles1 : tiles2;
   if (grid > most) grid = most;
-  if (dtype == 0) {
-    hipLaunchKernelGGL((decode_mlp_kernel<Bf16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar, phases);
-  } else {
-    hipLaunchKernelGGL((decode_mlp_kernel<Fp16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar, phases);
+  int slot = -1;
+  if (phases == 3) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    e = hipStreamIsCapturing(stream, &cap);
+    if (e != hipSuccess) return e;
+    if (cap != hipStreamCaptureStatusNone) return hipSuccess;
+    for (int i = 0; i < DEC_SLOTS && slot < 0; ++i) {
+      const int s = (int)((d->next + i) % DEC_SLOTS);
+      if (!d->used[s]) {
+        e = hipEventCreateWithFlags(&d->done[s], hipEventDisableTiming);
+        if (e != hipSuccess) return e;
+        slot = s;
+      } else if (hipEventQuery(d->done[s]) == hipSuccess) {
+        slot = s;
+      }
+    }
+    (void)hipGetLastError();  // hipErrorNotReady of the queries is not an error of this call
+    if (slot < 0) return hipSuccess;  // 64 single-launch forwards in flight
+    d->used[slot] = true;
+    d->next = (unsigned)slot + 1;
   }
-  return hipGetLastError();
+  unsigned* bar = d->bar + (slot < 0 ? 0 : slot) * 4;
+  const unsigned expected = (unsigned)grid + (test_unreachable ? 1u : 0u);
+  const unsigned spin_limit = test_unreachable ? 64u : DEC_SPIN_LIMIT;
+  if (dtype == 0) {
+    hipLaunchKernelGGL((decode_mlp_kernel<Bf16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar, phases,
+                       expected, spin_limit);
+  } else {
+    hipLaunchKernelGGL((decode_mlp_kernel<Fp16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar, phases,
+                       expected, spin_limit);
+  }
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  if (launched) *launched = true;
+  if (slot >= 0) e = hipEventRecord(d->done[slot], stream);
+  return e;
+}
+
+// Number of single-launch forwards on the current device whose device-wide barrier gave up since the last call
+// (their Y is incomplete); clears the marks. Synchronous copies: call it with no such forward in flight.
+hipError_t decode_barrier_failures(int* count) {
+  *count = 0;
+  std::lock_guard<std::mutex> lock(g_dec_mutex);
+  DecodeDevice* d = nullptr;
+  hipError_t e = decode_device(d);
+  if (e != hipSuccess) return e;
+  unsigned host[DEC_SLOTS * 4];
+  e = hipMemcpy(host, d->bar, sizeof(host), hipMemcpyDeviceToHost);
+  if (e != hipSuccess) return e;
+  const unsigned zero = 0;
+  for (int s = 0; s < DEC_SLOTS; ++s) {
+    if (host[s * 4 + 2] == 0) continue;
+    ++*count;
+    e = hipMemcpy(d->bar + s * 4 + 2, &zero, sizeof(zero), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 }  // namespace fsw

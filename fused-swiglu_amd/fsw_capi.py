@@ -34,6 +34,7 @@ PROTOTYPES = {
     "fsw_gateup_ws": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
     "fsw_strerror": (_cp, [_i]),
     "fsw_last_hip_error": (_i, []),
+    "fsw_decode_barrier_failures": (_i, []),
     "fsw_version": (_i, []),
     "fsw_set_variant": (_i, [_i, _i]),
     "fsw_variant_name": (_cp, [_i, _i, _i64, _i64, _i64]),
@@ -100,16 +101,45 @@ def _ld(t):
     return t.shape[1]
 
 
+def _check_operands(first, *others, out=None, out_shape=None, workspace=None):
+    """The guards of the PyTorch operator surface, for callers of the raw C ABI: 2-D device tensors with a unit
+    inner stride, all on one device; `out` of the same type with the expected shape; `workspace` a uint8 device
+    tensor. A transposed view passes a leading-dimension test and would be read as if it were row-major."""
+    import torch
+    for t in (first,) + others + ((out,) if out is not None else ()):
+        if t.dim() != 2:
+            raise FswError(E_SHAPE, "fsw: operands must be 2-D")
+        if not t.is_cuda:
+            raise FswError(E_DEVICE, "fsw: operands must be device tensors")
+        if t.device != first.device:
+            raise FswError(E_DEVICE, "fsw: operands live on different devices")
+        if t.shape[1] > 1 and t.stride(1) != 1:
+            raise FswError(E_LD, "fsw: operands must be contiguous in their last dimension")
+        if t.shape[0] > 1 and t.shape[1] > 0 and t.stride(0) < t.shape[1]:
+            raise FswError(E_LD, "fsw: overlapping rows")
+    if out is not None:
+        if out.dtype != first.dtype or tuple(out.shape) != tuple(out_shape):
+            raise FswError(E_SHAPE, "fsw: `out` must be a %s tensor of shape %s" % (first.dtype, tuple(out_shape)))
+    if workspace is not None:
+        if workspace.dtype != torch.uint8 or not workspace.is_cuda or workspace.device != first.device or \
+                not workspace.is_contiguous():
+            raise FswError(E_WORKSPACE, "fsw: workspace must be a contiguous uint8 tensor on the operands' device")
+
+
 def gateup(X, W13, out=None):
     """H[M, ff] = up * silu(gate) through fsw_gateup on the current stream. X [M,K], W13 [2ff,K] device tensors."""
     import torch
     code = dtype_code(X)
     if W13.dtype != X.dtype:
         raise FswError(E_DTYPE, "fsw: X and W13 differ in element type")
+    _check_operands(X, W13)
     M, K = X.shape
     N = W13.shape[0]
+    if W13.shape[1] != K:
+        raise FswError(E_SHAPE, "fsw: X is [M, K] and W13 is [2 ff, K]: K differs")
     if out is None:
         out = torch.empty((M, N // 2), dtype=X.dtype, device=X.device)
+    _check_operands(X, out=out, out_shape=(M, N // 2))
     nbytes = lib().fsw_gateup_workspace_bytes(code, M, N, K)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device) if nbytes else None
     with torch.cuda.device(X.device):
@@ -124,10 +154,14 @@ def down(H, W2, out=None):
     code = dtype_code(H)
     if W2.dtype != H.dtype:
         raise FswError(E_DTYPE, "fsw: H and W2 differ in element type")
+    _check_operands(H, W2)
     M, FF = H.shape
     D = W2.shape[0]
+    if W2.shape[1] != FF:
+        raise FswError(E_SHAPE, "fsw: H is [M, FF] and W2 is [D, FF]: FF differs")
     if out is None:
         out = torch.empty((M, D), dtype=H.dtype, device=H.device)
+    _check_operands(H, out=out, out_shape=(M, D))
     nbytes = lib().fsw_down_workspace_bytes(code, M, D, FF)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=H.device) if nbytes else None
     with torch.cuda.device(H.device):
@@ -149,12 +183,16 @@ def mlp(X, W13, W2, out=None, workspace=None):
     code = dtype_code(X)
     if W13.dtype != X.dtype or W2.dtype != X.dtype:
         raise FswError(E_DTYPE, "fsw: X, W13 and W2 differ in element type")
+    _check_operands(X, W13, W2)
     M, D = X.shape
     FF = W13.shape[0] // 2
+    if W13.shape[1] != D or tuple(W2.shape) != (D, FF):
+        raise FswError(E_SHAPE, "fsw: X is [M, d], W13 is [2 ff, d] and W2 is [d, ff]")
     if out is None:
         out = torch.empty((M, D), dtype=X.dtype, device=X.device)
     if workspace is None:
         workspace = mlp_workspace(X, FF)
+    _check_operands(X, out=out, out_shape=(M, D), workspace=workspace)
     with torch.cuda.device(X.device):
         check(lib().fsw_mlp(code, M, D, FF, X.data_ptr(), _ld(X), W13.data_ptr(), _ld(W13), W2.data_ptr(), _ld(W2),
                             out.data_ptr(), _ld(out), workspace.data_ptr(), workspace.numel(), _stream(X)))
@@ -180,6 +218,7 @@ def _blocked_empty(rows, k, like):
 def block_rows(A, kind="rows"):
     """Row-major device matrix -> Blocked. kind: "rows" (X, H, W2) or "w13" (up/gate rows de-interleaved per panel)."""
     import torch
+    _check_operands(A)
     rows, k = A.shape
     out = _blocked_empty(rows, k, A)
     fn = {"rows": lib().fsw_block_rows, "w13": lib().fsw_prepack_w13, "w2": lib().fsw_prepack_w2}[kind]
@@ -234,6 +273,14 @@ def down_blocked(Hb, W2, out=None):
 
 def set_variant(family, variant):
     check(lib().fsw_set_variant(family, variant))
+
+
+def decode_barrier_failures():
+    """Single-launch decode forwards whose device-wide barrier gave up since the last call (synchronous)."""
+    n = lib().fsw_decode_barrier_failures()
+    if n < 0:
+        check(n)
+    return n
 
 
 def variant_name(family, dtype, M, n, k):

@@ -13,7 +13,11 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); launches are
  *     asynchronous, nothing here synchronises;
  *   - the return value is FSW_OK (0) or a negative FSW_E_* code; nothing throws or aborts;
- *   - the fsw_validate_* functions touch no GPU API and can be called on a machine without one.
+ *   - the fsw_validate_* functions touch no GPU API and can be called on a machine without one;
+ *   - entry points are re-entrant: there is no process-wide mutable state apart from caches of device properties
+ *     (filled atomically), so any number of host threads may call them on any streams at the same time;
+ *   - the library links the HIP runtime (libamdhip64). A process must hold ONE copy of it: inside a PyTorch-ROCm
+ *     process, load torch (which brings its own) BEFORE this library, or launches fail with FSW_E_DEVICE.
  *
  * Weight formats (identical to the reference's):
  *   W13 [N = 2*ff, K] row-major, K-contiguous, rows interleaved: row 2j   = "up"  (linear) operand,
@@ -149,17 +153,30 @@ FSW_API int fsw_last_hip_error(void);
 FSW_API int fsw_version(void);
 
 /*
- * Kernel-selection override for tuning and tests. family: 0 = gate/up, 1 = down; variant < 0 restores the
- * automatic choice by shape; variant 100 is the weight-streaming kernel (honoured for M <= 64; the
- * dispatcher itself picks it up to 16 .. 48 rows, the larger the weights the fewer); variant 102 is the
+ * Kernel-selection override for tests and tuning, PER CALLING THREAD (thread-local): it changes the kernel choice
+ * of later calls made by the same thread only, so a thread's fsw_*_workspace_bytes() queries and the launches
+ * that follow them always agree. family: 0 = gate/up, 1 = down; variant < 0 restores the automatic choice by
+ * shape; 0 .. 5 force one tiled kernel (dma_128x128, dma_128x256, dma_128x192, dma8w_128x256, dma_128x64,
+ * pair16_256x256; a forced kernel runs unsplit and needs no scratch); 100 is the weight-streaming kernel (honoured
+ * for M <= 64; the dispatcher itself picks it up to 16 .. 48 rows, the larger the weights the fewer); 102 is the
  * persistent streaming kernel (honoured for M <= 16; automatic only for d * ff >= 2^27); family 0 variant 101
- * makes fsw_mlp run M <= 16 as one persistent launch (gate/up, device-wide barrier, down) instead of two launches.
- * family 2 sets the raster band height of the tiled kernels instead (0 = per-kernel default).
- * family 3 picks the kernel behind the blocked entry points for row-major weights: 2 = pair ring on
- * v_mfma_f32_16x16x32 (default), 1 = pair ring on v_mfma_f32_32x32x16, 0 = plain ring.
- * Returns FSW_E_VARIANT for unknown ids. Process-wide and not thread-safe against concurrent launches.
+ * makes fsw_mlp run M <= 16 as ONE persistent launch (gate/up, device-wide barrier, down) instead of two launches
+ * -- see fsw_decode_barrier_failures(); 103 is 101 with a barrier that cannot complete (failure-path test).
+ * Returns FSW_E_VARIANT for unknown ids.
  */
 FSW_API int fsw_set_variant(int family, int variant);
+
+/*
+ * The single-launch decode forward (fsw_set_variant(0, 101)) synchronises its workgroups with a device-wide barrier,
+ * which completes only if all of them are resident at once. The wait is bounded: when other work holds compute units
+ * the kernel gives up, skips the down projection (Y is left incomplete, never computed from a partial H) and marks
+ * its barrier slot. This call returns how many such launches there were on the current device since it was last
+ * called and clears the marks, or a negative FSW_E_* code. It copies synchronously: call it after synchronising the
+ * stream, with no single-launch forward in flight. A caller that opts into variant 101 must check it before using Y.
+ * With 64 single-launch forwards in flight, or on a stream that is being captured into a graph, fsw_mlp runs the
+ * two-launch path instead. No counterpart in the reference.
+ */
+FSW_API int fsw_decode_barrier_failures(void);
 
 /* Name of the kernel variant the dispatcher picks for this shape (static storage); "splitk_<kernel>" when the
  * down projection splits K (family 1; K_or_FF decides). */

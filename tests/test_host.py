@@ -93,6 +93,9 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu(capi):
     assert L.fsw_mlp_workspace_bytes(0, 0, 16, 8) == 0
     assert L.fsw_set_variant(0, 12345) == capi.E_VARIANT
     assert L.fsw_set_variant(7, 0) == capi.E_VARIANT
+    assert L.fsw_set_variant(2, 4) == capi.E_VARIANT and L.fsw_set_variant(0, 6) == capi.E_VARIANT
+    assert L.fsw_mlp(7, 4, 16, 8, 0x1000, 16, 0x2000, 16, 0x3000, 8, 0x4000, 16, None, 0, None) == capi.E_DTYPE
+    assert L.fsw_mlp(0, 4, 0, 8, 0x1000, 0, None, 0, None, 8, None, 0, None, 0, None) == capi.OK  # D = 0: no Y
     assert L.fsw_set_variant(0, -1) == capi.OK
     with pytest.raises(capi.FswError) as ei:
         capi.check(capi.E_ALIGN)
@@ -123,6 +126,7 @@ def test_variant_choice_by_regime(capi):
         assert name(0, 4, 64, 32) == "decode_stream" and name(0, 17, 64, 32) == "skinny"
         assert name(1, 16, 8192, 28672) == "skinny"          # forced weight-streaming kernel wins over the size rule
         assert L.fsw_set_variant(1, 101) == capi.E_VARIANT   # the single-launch form is a family-0 (fsw_mlp) option
+        assert L.fsw_set_variant(1, 103) == capi.E_VARIANT
     finally:
         L.fsw_set_variant(0, -1)
         L.fsw_set_variant(1, -1)
@@ -143,6 +147,47 @@ def test_variant_choice_by_regime(capi):
     assert ws(0, 8192, 4096, 14336) == L.fsw_blocked_bytes(8192, 14336) == 8192 * 14336 * 2
     assert ws(0, 3000, 4096, 14336) == L.fsw_blocked_bytes(3000, 14336) and ws(0, 16, 4096, 14336) == 0
     assert capi.lib().fsw_mlp_workspace_bytes(0, 256, 4096, 14336) == 256 * 14336 * 2 + ws(0, 256, 4096, 14336)
+
+
+def test_variant_override_is_per_thread(capi):
+    """fsw_set_variant is thread-local: another thread's override neither shows here nor changes what this thread's
+    workspace query and launch agree on."""
+    import threading
+    L = capi.lib()
+    name = lambda: capi.variant_name(1, 0, 200, 512, 4096)
+    assert name() == "splitk_dma_128x128" and L.fsw_down_workspace_bytes(0, 200, 512, 4096) > 0
+    seen = {}
+
+    def other():
+        assert L.fsw_set_variant(1, 0) == capi.OK
+        seen["name"] = name()
+        seen["ws"] = L.fsw_down_workspace_bytes(0, 200, 512, 4096)
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    assert seen == {"name": "dma_128x128", "ws": 0}
+    assert name() == "splitk_dma_128x128" and L.fsw_down_workspace_bytes(0, 200, 512, 4096) > 0
+
+
+def test_ctypes_wrappers_refuse_views_the_c_abi_would_misread(capi):
+    """The raw C ABI takes pointers and leading dimensions; a transposed view passes its leading-dimension test and
+    would be read as if it were row-major. The wrappers apply the guards of the PyTorch operator surface before any
+    GPU call (CPU tensors are refused here as well: there is no CPU path)."""
+    X = torch.zeros(16, 16, dtype=torch.bfloat16)
+    W = torch.zeros(32, 16, dtype=torch.bfloat16)
+    with pytest.raises(capi.FswError) as ei:
+        capi.gateup(X, W)
+    assert ei.value.code == capi.E_DEVICE
+    meta = lambda *shape: torch.empty(*shape, dtype=torch.bfloat16, device="meta")
+    with pytest.raises(capi.FswError):
+        capi._check_operands(meta(16, 16).t())
+    Xt = torch.empty(16, 32, dtype=torch.bfloat16).t()   # [32, 16] with strides (1, 32)
+    with pytest.raises(capi.FswError) as ei:
+        capi._check_operands(Xt)
+    assert ei.value.code in (capi.E_LD, capi.E_DEVICE)
+    with pytest.raises(capi.FswError):
+        capi._check_operands(torch.zeros(4, 4, 4, dtype=torch.bfloat16))
 
 
 def test_packers_follow_the_reference_interleave():

@@ -93,7 +93,7 @@ def test_gateup_any_ff(capi, shape, dtype):
     assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "H %s" % (shape,))
 
 
-@pytest.mark.parametrize("variant", list(range(19)))
+@pytest.mark.parametrize("variant", list(range(6)))
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_every_tiled_variant(capi, variant, dtype):
     try:
@@ -207,6 +207,59 @@ def test_single_launch_decode_forward(capi, M, dtype):
             assert torch.equal(r, Y1)
         oracle.assert_parity(Yb, oracle.ref_mlp(inp_b["X"], inp["W13"], inp["W2"], torch.float64), "fused mlp, second input %s" % ((M, d, ff),))
         assert torch.equal(Ya, Y1)
+    torch.cuda.synchronize()
+    assert capi.decode_barrier_failures() == 0
+
+
+def test_single_launch_decode_reports_a_failed_barrier(capi):
+    """Variant 103 is the single-launch forward with a device-wide barrier that waits for one arrival more than the
+    grid has and polls 64 times only: every workgroup takes the give-up path. The kernel must end normally, write NO
+    Y (the down projection is skipped, not run on a partial H), leave the barrier slot reusable, and the failure must
+    be visible through fsw_decode_barrier_failures() exactly once."""
+    M, d, ff = 8, 1000, 264
+    inp = fsw_weights.make_inputs(M, d, ff, torch.bfloat16, seed=5, x_scale=0.5)
+    g = to_dev(inp)
+    ws = capi.mlp_workspace(g["X"], ff)
+    torch.cuda.synchronize()
+    assert capi.decode_barrier_failures() == 0
+    Y = torch.full((M, d), 7.0, dtype=torch.bfloat16, device=DEV)
+    try:
+        capi.set_variant(0, 103)
+        capi.mlp(g["X"], g["W13"], g["W2"], out=Y, workspace=ws)
+        torch.cuda.synchronize()
+    finally:
+        capi.set_variant(0, -1)
+    assert (Y.float() == 7.0).all(), "a failed single launch must not write Y"
+    assert capi.decode_barrier_failures() == 1
+    assert capi.decode_barrier_failures() == 0
+    # the gate/up half did run, and the slot works again: 70 good launches walk over all 64 slots
+    H = ws[: M * ff * 2].view(torch.bfloat16).view(M, ff)
+    assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), torch.bfloat16, "H of a failed launch")
+    ref = oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64)
+    try:
+        capi.set_variant(0, 101)
+        for _ in range(70):
+            Y.fill_(7.0)
+            capi.mlp(g["X"], g["W13"], g["W2"], out=Y, workspace=ws)
+        torch.cuda.synchronize()
+    finally:
+        capi.set_variant(0, -1)
+    oracle.assert_parity(Y, ref, "single launch after a failed one")
+    assert capi.decode_barrier_failures() == 0
+    # on a capturing stream the single launch is refused and the two-launch path is recorded instead
+    graph = torch.cuda.CUDAGraph()
+    Yg = torch.empty_like(Y)
+    try:
+        capi.set_variant(0, 101)
+        with torch.cuda.graph(graph):
+            capi.mlp(g["X"], g["W13"], g["W2"], out=Yg, workspace=ws)
+    finally:
+        capi.set_variant(0, -1)
+    for _ in range(2):
+        Yg.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Yg, capi.mlp(g["X"], g["W13"], g["W2"]))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -230,7 +283,7 @@ def test_split_k_down_projection(capi, dtype):
         ref = oracle.ref_down(H[rows.to(DEV)].cpu(), inp["W2"], torch.float64)
         assert_one_rounding(Y[rows.to(DEV)], ref, dtype, "split-K Y %s (scratch %d B)" % ((M, d, ff), nbytes))
         try:
-            capi.set_variant(1, 7)  # same tile shape, no split
+            capi.set_variant(1, 0)  # 128 x 128 tiles, no split
             Y1 = capi.down(H, g["W2"])
         finally:
             capi.set_variant(1, -1)
@@ -262,6 +315,29 @@ def test_empty_and_degenerate_problems(capi):
     H = capi.gateup(torch.empty(4, 0, device=DEV, dtype=bf), torch.empty(16, 0, device=DEV, dtype=bf),
                     out=torch.full((4, 8), 7.0, device=DEV, dtype=bf))
     assert H.abs().max().item() == 0.0
+    # the same through the tiled kernels (M > 64): K = 0 writes zeros, ff = 0 gives Y = 0, D = 0 needs no Y at all
+    for M in (70, 300):
+        H = capi.gateup(torch.empty(M, 0, device=DEV, dtype=bf), torch.empty(16, 0, device=DEV, dtype=bf),
+                        out=torch.full((M, 8), 7.0, device=DEV, dtype=bf))
+        assert H.abs().max().item() == 0.0
+        Xm = torch.randn(M, 64, device=DEV).to(bf)
+        Y = capi.mlp(Xm, torch.empty(0, 64, device=DEV, dtype=bf), torch.empty(64, 0, device=DEV, dtype=bf),
+                     out=torch.full((M, 64), 7.0, device=DEV, dtype=bf))
+        assert Y.abs().max().item() == 0.0
+        L = capi.lib()
+        assert L.fsw_mlp(0, M, 0, 8, Xm.data_ptr(), 64, None, 0, None, 8, None, 0, None, 0, None) == capi.OK
+    # a forced tiled kernel runs unsplit and asks for no scratch
+    try:
+        capi.set_variant(1, 0)
+        assert capi.lib().fsw_down_workspace_bytes(0, 200, 512, 4096) == 0
+        Hh = torch.randn(200, 4096, device=DEV).to(bf)
+        W2 = torch.randn(512, 4096, device=DEV).to(bf)
+        Yf = torch.empty(200, 512, device=DEV, dtype=bf)
+        assert capi.lib().fsw_down(0, 200, 512, 4096, Hh.data_ptr(), 4096, W2.data_ptr(), 4096, Yf.data_ptr(), 512,
+                                   None, 0, torch.cuda.current_stream().cuda_stream) == capi.OK
+    finally:
+        capi.set_variant(1, -1)
+    assert_one_rounding(Yf, Hh.cpu().double() @ W2.cpu().double().T, bf, "forced unsplit down", slack=0.25)
 
 
 def test_even_odd_convention_on_device(capi):
@@ -488,8 +564,7 @@ def test_blocked_kernels_against_oracle(capi, dtype, prepacked):
 
 def test_blocked_kernels_take_strided_row_major_operands(capi):
     """Row strides larger than the row (column slices of wider tensors) for X into fsw_block_rows, for the
-    row-major W13 / W2 of the pair-ring kernels and for Y; also the other kernel behind the blocked entry points
-    (plain ring, fsw_set_variant(3, 0); pair ring on 32x32x16 MFMAs, (3, 1)) must give the same bits."""
+    row-major W13 / W2 of the blocked entry points and for Y."""
     M, d, ff = 300, 1096, 520
     dtype = torch.bfloat16
     inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=123, x_scale=0.5)
@@ -502,14 +577,6 @@ def test_blocked_kernels_take_strided_row_major_operands(capi):
     Y = capi.down_blocked(Hb, W2, out=Ybig[:, :d])
     oracle.assert_parity(Y, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64), "blocked, strided operands")
     assert torch.isnan(Ybig[:, d:]).all()
-    for mode in (0, 1):  # plain ring, pair ring on 32x32x16 MFMAs; the default (2) is the pair ring on 16x16x32
-        try:
-            capi.set_variant(3, mode)
-            Hb2 = capi.gateup_blocked(Xb, W13)
-            Y2 = capi.down_blocked(Hb2, W2)
-        finally:
-            capi.set_variant(3, 2)
-        assert torch.equal(capi.unblock(Hb2), capi.unblock(Hb)) and torch.equal(Y2, Y), "mode %d" % mode
 
 
 def test_mlp_large_tile_regime_uses_blocked_path(capi):
