@@ -36,6 +36,8 @@ PROTOTYPES = {
     "fsw_last_hip_error": (_i, []),
     "fsw_decode_barrier_failures": (_i, []),
     "fsw_version": (_i, []),
+    "fsw_probe_mfma": (_i, [_i, _i, _vp, _vp, _i, _vp]),
+    "fsw_probe_read": (_i, [_vp, _sz, _vp, _i, _vp]),
     "fsw_set_variant": (_i, [_i, _i]),
     "fsw_variant_name": (_cp, [_i, _i, _i64, _i64, _i64]),
 }

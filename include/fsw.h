@@ -178,6 +178,17 @@ FSW_API int fsw_set_variant(int family, int variant);
  */
 FSW_API int fsw_decode_barrier_failures(void);
 
+/*
+ * Measurement kernels (no counterpart in the reference): what this board sustains with nothing else in the way,
+ * for the benchmark to print beside its roofline fractions.
+ * fsw_probe_mfma: `workgroups` x 4 waves each issue iters x 64 v_mfma_f32_16x16x32 from registers (the prefill
+ *   kernel's accumulator shape); = workgroups * 4 * iters * 64 * 16384 FLOP. `operands`: 16 KB of device data in the
+ *   element type (its values set the power draw), 16-byte aligned; `out`: workgroups * 1 KB of device scratch.
+ * fsw_probe_read: streams `bytes` (a multiple of 16) from `src` once with non-temporal 16-byte loads; `out`: 4 bytes.
+ */
+FSW_API int fsw_probe_mfma(int dtype, int iters, const void* operands, void* out, int workgroups, void* stream);
+FSW_API int fsw_probe_read(const void* src, size_t bytes, void* out, int workgroups, void* stream);
+
 /* Name of the kernel variant the dispatcher picks for this shape (static storage); "splitk_<kernel>" when the
  * down projection splits K (family 1; K_or_FF decides). */
 FSW_API const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, int64_t K_or_FF);
