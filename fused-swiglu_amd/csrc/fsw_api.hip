@@ -158,6 +158,7 @@ const char* fsw_strerror(int code) {
     case FSW_E_LAUNCH: return "fsw: the HIP runtime rejected the kernel launch";
     case FSW_E_DEVICE: return "fsw: the current device is not a gfx950 GPU";
     case FSW_E_VARIANT: return "fsw: unknown kernel variant";
+    case FSW_E_STATIC_LIMIT: return "fsw: the problem needs more scratch than the library's static 64 MiB; use fsw_mlp";
     default: return "fsw: unknown error code";
   }
 }
@@ -548,6 +549,52 @@ int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t 
             const void* W2, int64_t ldw2, void* Y, int64_t ldy, void* workspace, size_t workspace_bytes,
             void* stream) {
   return mlp_impl(dtype, M, D, FF, X, ldx, W13, ldw13, W2, ldw2, Y, ldy, workspace, workspace_bytes, stream, true);
+}
+
+// ---- the entry point that allocates nothing ------------------------------------------------------------------
+// fsw_mlp with its workspace inside the library: a file-scope device array that every GPU the library runs on
+// holds until the process ends. The array's name is a host-side stand-in, not a device address; its address on a
+// device comes from hipGetSymbolAddress, asked once per device with that device current, and only that pointer is
+// handed to kernels.
+#define FSW_STATIC_SCRATCH_BYTES (64u << 20)
+static __device__ __align__(256) unsigned char scratch[FSW_STATIC_SCRATCH_BYTES];
+
+// device address of `scratch` on the current device (looked up on the first call per device, then cached)
+static int static_scratch_ptr(void** out) {
+  static std::atomic<void*> ptr_of_device[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= 64) {
+    g_last_hip_error = (int)e;
+    return FSW_E_DEVICE;
+  }
+  void* p = ptr_of_device[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      g_last_hip_error = (int)e;
+      return FSW_E_LAUNCH;
+    }
+    ptr_of_device[dev].store(p, std::memory_order_release);  // racing first calls on one device store the same address
+  }
+  *out = p;
+  return FSW_OK;
+}
+
+size_t fsw_mlp_static_max_bytes(void) { return FSW_STATIC_SCRATCH_BYTES; }
+
+int fsw_mlp_static(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, int64_t ldx, const void* W13,
+                   int64_t ldw13, const void* W2, int64_t ldw2, void* Y, int64_t ldy, void* stream) {
+  if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
+  if (M < 0 || D < 0 || FF < 0 || M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM / 2) return FSW_E_SHAPE;
+  if (M == 0 || D == 0) return FSW_OK;
+  if (fsw_mlp_workspace_bytes(dtype, M, D, FF) > FSW_STATIC_SCRATCH_BYTES) return FSW_E_STATIC_LIMIT;
+  const int drc = check_device();
+  if (drc != FSW_OK) return drc;
+  void* ws = nullptr;
+  const int rc = static_scratch_ptr(&ws);
+  if (rc != FSW_OK) return rc;
+  return mlp_impl(dtype, M, D, FF, X, ldx, W13, ldw13, W2, ldw2, Y, ldy, ws, FSW_STATIC_SCRATCH_BYTES, stream, false);
 }
 
 }  // extern "C"

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(HERE, "libfsw_hip.so")
 
 BF16, FP16 = 0, 1
 OK = 0
-E_NULL, E_DTYPE, E_SHAPE, E_LD, E_ALIGN, E_WORKSPACE, E_LAUNCH, E_DEVICE, E_VARIANT = range(-1, -10, -1)
+E_NULL, E_DTYPE, E_SHAPE, E_LD, E_ALIGN, E_WORKSPACE, E_LAUNCH, E_DEVICE, E_VARIANT, E_STATIC_LIMIT = range(-1, -11, -1)
 
 # name -> (restype, argtypes); the list the loader test checks against include/fsw.h
 _i, _i64, _vp, _sz, _cp = ctypes.c_int, ctypes.c_int64, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_char_p
@@ -24,6 +24,8 @@ PROTOTYPES = {
     "fsw_down": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
     "fsw_mlp_workspace_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "fsw_mlp": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
+    "fsw_mlp_static_max_bytes": (_sz, []),
+    "fsw_mlp_static": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "fsw_blocked_bytes": (_sz, [_i64, _i64]),
     "fsw_block_rows": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
     "fsw_prepack_w13": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
@@ -198,6 +200,24 @@ def mlp(X, W13, W2, out=None, workspace=None):
     with torch.cuda.device(X.device):
         check(lib().fsw_mlp(code, M, D, FF, X.data_ptr(), _ld(X), W13.data_ptr(), _ld(W13), W2.data_ptr(), _ld(W2),
                             out.data_ptr(), _ld(out), workspace.data_ptr(), workspace.numel(), _stream(X)))
+    return out
+
+
+def mlp_static(X, W13, W2, out):
+    """fsw_mlp_static: the forward with the library's own static scratch; `out` is required (nothing is allocated)."""
+    import torch
+    code = dtype_code(X)
+    if W13.dtype != X.dtype or W2.dtype != X.dtype:
+        raise FswError(E_DTYPE, "fsw: X, W13 and W2 differ in element type")
+    _check_operands(X, W13, W2)
+    M, D = X.shape
+    FF = W13.shape[0] // 2
+    if W13.shape[1] != D or tuple(W2.shape) != (D, FF):
+        raise FswError(E_SHAPE, "fsw: X is [M, d], W13 is [2 ff, d] and W2 is [d, ff]")
+    _check_operands(X, out=out, out_shape=(M, D))
+    with torch.cuda.device(X.device):
+        check(lib().fsw_mlp_static(code, M, D, FF, X.data_ptr(), _ld(X), W13.data_ptr(), _ld(W13), W2.data_ptr(),
+                                   _ld(W2), out.data_ptr(), _ld(out), _stream(X)))
     return out
 
 

@@ -53,6 +53,7 @@ extern "C" {
 #define FSW_E_LAUNCH     -7   /* the HIP runtime rejected a launch (see fsw_last_hip_error) */
 #define FSW_E_DEVICE     -8   /* the current device is not a gfx950 GPU */
 #define FSW_E_VARIANT    -9   /* unknown kernel variant requested through fsw_set_variant */
+#define FSW_E_STATIC_LIMIT -10 /* fsw_mlp_static: the shape needs more scratch than the library's static array */
 
 /*
  * Host-only argument validation of fsw_gateup (replaces the dtype TORCH_CHECKs of swiglu.cu:475-480 and adds
@@ -108,6 +109,22 @@ FSW_API int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF,
             const void* X, int64_t ldx, const void* W13, int64_t ldw13,
             const void* W2, int64_t ldw2, void* Y, int64_t ldy,
             void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * fsw_mlp for callers that cannot allocate device memory at all (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments without the workspace, same kernels, same result bit for
+ * bit. No counterpart in the reference. The scratch (H, split-K partials, the blocked copy of X) lives in a static
+ * device array of fsw_mlp_static_max_bytes() = 64 MiB inside the library, which every GPU the library runs on holds
+ * until the process ends; shapes whose fsw_mlp_workspace_bytes() exceed it return FSW_E_STATIC_LIMIT (it covers
+ * decode and small batches: at d = 4096, ff = 14336 every M <= 468). The call itself allocates and frees nothing;
+ * the first call on a device looks the array's address up (make it outside graph capture). All calls on one GPU share
+ * the one array: calls that overlap in time on the same GPU (different streams, concurrent graph replays) race on
+ * it and must be serialised by the caller. The single-launch decode option of fsw_set_variant is ignored here.
+ */
+FSW_API size_t fsw_mlp_static_max_bytes(void);
+FSW_API int fsw_mlp_static(int dtype, int64_t M, int64_t D, int64_t FF,
+                           const void* X, int64_t ldx, const void* W13, int64_t ldw13,
+                           const void* W2, int64_t ldw2, void* Y, int64_t ldy, void* stream);
 
 /* Text for an FSW_E_* code (static storage, never NULL). */
 FSW_API const char* fsw_strerror(int code);
