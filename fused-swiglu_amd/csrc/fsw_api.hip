@@ -20,6 +20,7 @@ constexpr int VARIANT_SKINNY = 100;          // id of the weight-streaming kerne
 constexpr int VARIANT_DECODE_STREAM = 102;   // M <= 16: the streaming kernel of kernels_decode.hip, one phase per launch
 constexpr int VARIANT_DECODE_FUSED = 101;    // fsw_mlp only: single-launch decode forward (family 0)
 constexpr int VARIANT_DECODE_FUSED_FAIL = 103;  // 101 with a device-wide barrier that cannot complete (failure-path test)
+constexpr int VARIANT_STREAM_SPLIT = 104;    // family 1, fsw_mlp only: split-K streaming down projection for M <= 32
 constexpr int64_t MAX_DIM = 1LL << 30;       // every size is cast to int inside the kernels
 constexpr int64_t MAX_LD = 1LL << 21;        // keeps tile-relative byte offsets below 2^31
 
@@ -101,7 +102,8 @@ int64_t decode_rows(int family, int64_t np, int64_t k) {
 
 int resolve_variant(int family, int64_t m, int64_t np, int64_t k) {
   const int forced = g_forced_variant[family];
-  if (forced == VARIANT_DECODE_FUSED || forced == VARIANT_DECODE_FUSED_FAIL || forced == VARIANT_DECODE_STREAM)
+  if (forced == VARIANT_DECODE_FUSED || forced == VARIANT_DECODE_FUSED_FAIL || forced == VARIANT_DECODE_STREAM ||
+      forced == VARIANT_STREAM_SPLIT)
     return m <= 64 ? VARIANT_SKINNY : pick_tiled(family, m, np);
   if (forced >= 0 && !(forced == VARIANT_SKINNY && m > 64)) return forced;
   if (m <= decode_rows(family, np, k)) {  // decode and small batches: weight streaming, HBM bound
@@ -177,6 +179,7 @@ int fsw_set_variant(int family, int variant) {
   if (family < 0 || family > 1) return FSW_E_VARIANT;
   if (variant >= 0 && variant != VARIANT_SKINNY && variant != VARIANT_DECODE_STREAM &&
       !(family == 0 && (variant == VARIANT_DECODE_FUSED || variant == VARIANT_DECODE_FUSED_FAIL)) &&
+      !(family == 1 && variant == VARIANT_STREAM_SPLIT) &&
       variant >= fsw::tiled_variant_count())
     return FSW_E_VARIANT;
   g_forced_variant[family] = variant < 0 ? -1 : variant;
@@ -185,8 +188,14 @@ int fsw_set_variant(int family, int variant) {
 
 static bool down_reblock_wanted(int64_t M, int64_t D, int64_t FF);
 
+static fsw::StreamPlan mlp_stream_plan(int64_t M, int64_t D, int64_t FF);
+
 const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, int64_t K_or_FF) {
   (void)dtype;
+  if (family == 2) {  // the down projection as fsw_mlp runs it
+    if (mlp_stream_plan(M, N_or_D, K_or_FF).splits > 1) return "stream_split";
+    family = 1;
+  }
   if (family < 0 || family > 1) return "invalid";
   const int v = resolve_variant(family, M, N_or_D, K_or_FF);
   if (v == VARIANT_SKINNY) return decode_stream_wanted(family, M, N_or_D, K_or_FF) ? "decode_stream" : "skinny";
@@ -235,8 +244,9 @@ int fsw_validate_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H
   return FSW_OK;
 }
 
-int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13, int64_t ldw,
-               void* H, int64_t ldh, void* stream) {
+// zero_words / n_zero_words: see GemmArgs (only the decode-regime kernels honour them; the caller checks that)
+static int gateup_impl(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13,
+                       int64_t ldw, void* H, int64_t ldh, void* stream, unsigned* zero_words, int n_zero_words) {
   const int rc = fsw_validate_gateup(dtype, M, N, K, X, ldx, W13, ldw, H, ldh);
   if (rc != FSW_OK) return rc;
   if (M == 0 || N == 0) return FSW_OK;
@@ -252,6 +262,8 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
   a.np = (int)N;
   a.nq = (int)M;
   a.k = (int)K;
+  a.zero_words = zero_words;
+  a.n_zero_words = n_zero_words;
   const int v = resolve_variant(0, M, N, K);
   if (v == VARIANT_SKINNY) {
     if (decode_stream_wanted(0, M, N, K)) {  // at most 16 rows: one 8-wave workgroup per CU, X held in registers
@@ -270,6 +282,33 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
     return finish(fsw::launch_skinny(dtype, true, a, nullptr, (hipStream_t)stream));
   }
   return finish(fsw::launch_tiled(v, dtype, true, a, (hipStream_t)stream));
+}
+
+int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13, int64_t ldw,
+               void* H, int64_t ldh, void* stream) {
+  return gateup_impl(dtype, M, N, K, X, ldx, W13, ldw, H, ldh, stream, nullptr, 0);
+}
+
+// Inside fsw_mlp the down projection of up to 32 activation rows runs the split-K streaming kernel when (i) the
+// gate/up product before it runs a kernel that zeroes the ticket counters (skinny_kernel or the 128 x 64 tiled
+// kernel), (ii) the down projection is in the weight-streaming regime and (iii) the shape is large enough for the
+// saved H traffic to matter (stream_split_plan) -- or when variant 104 forces it (then any shape it supports).
+static fsw::StreamPlan mlp_stream_plan(int64_t M, int64_t D, int64_t FF) {
+  const fsw::StreamPlan none = {0, 0, 0, 0};
+  if (M < 1 || M > 32 || D <= 0 || FF <= 0 || D > MAX_DIM || FF > MAX_DIM / 2) return none;
+  const int f1 = g_forced_variant[1];
+  if (f1 >= 0 && f1 != VARIANT_STREAM_SPLIT) return none;
+  const int f0 = g_forced_variant[0];
+  if (f0 == VARIANT_DECODE_FUSED || f0 == VARIANT_DECODE_FUSED_FAIL) return none;
+  const int v0 = resolve_variant(0, M, 2 * FF, D);
+  const bool zeroes = (v0 == VARIANT_SKINNY && !decode_stream_wanted(0, M, 2 * FF, D)) || v0 == V_128x64;
+  if (!zeroes) return none;
+  if (f1 == VARIANT_STREAM_SPLIT) return fsw::stream_split_plan((int)D, (int)M, (int)FF, true);
+  if (!streams_weights(1, M, D, FF) || decode_stream_wanted(1, M, D, FF)) return none;
+  return fsw::stream_split_plan((int)D, (int)M, (int)FF, false);
+}
+static size_t stream_scratch_bytes(const fsw::StreamPlan& p) {
+  return (p.partial_bytes + (size_t)p.ticket_words * 4 + 255) & ~(size_t)255;
 }
 
 // Row-major H in the large-tile regime: with scratch for a blocked copy of H the down projection runs the pair-ring
@@ -388,6 +427,7 @@ int fsw_prepack_w2(int dtype, int64_t D, int64_t FF, const void* W2, int64_t ldw
 
 int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* Xb, const void* W13, int64_t ldw,
                        int w_blocked, void* Hb, int64_t ldh, void* stream) {
+
   if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
   if (M < 0 || N < 0 || K < 0 || (N & 1) || M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return FSW_E_SHAPE;
   if (M == 0 || N == 0) return FSW_OK;
@@ -477,6 +517,8 @@ static size_t h_bytes(int64_t M, int64_t FF) {
 size_t fsw_mlp_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
   if (M <= 0 || D <= 0 || FF <= 0) return 0;
   if (blocked_regime(M, D, FF)) return (size_t)fsw::blocked_bytes(M, FF) + (size_t)fsw::blocked_bytes(M, D);
+  const fsw::StreamPlan sp = mlp_stream_plan(M, D, FF);
+  if (sp.splits > 1) return h_bytes(M, FF) + stream_scratch_bytes(sp);  // [H row-major][partials][ticket counters]
   // otherwise [H row-major][split-K scratch of the down projection][X blocked, when gate/up alone runs large tiles]
   return h_bytes(M, FF) + ((fsw_down_workspace_bytes(dtype, M, D, FF) + 255) & ~(size_t)255) +
          fsw_gateup_workspace_bytes(dtype, M, 2 * FF, D);
@@ -538,6 +580,23 @@ static int mlp_impl(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, 
     return fsw_down_blocked(dtype, M, D, FF, Hb, W2, ldw2, 0, Y, ldy, stream);
   }
   unsigned char* ws2 = (unsigned char*)workspace + h_bytes(M, FF);
+  const fsw::StreamPlan sp = mlp_stream_plan(M, D, FF);
+  if (sp.splits > 1) {  // decode: the gate/up kernel zeroes the ticket counters of the split-K streaming down projection
+    unsigned* tickets = (unsigned*)(ws2 + sp.partial_bytes);
+    rc = gateup_impl(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF, stream, tickets, sp.ticket_words);
+    if (rc != FSW_OK) return rc;
+    fsw::GemmArgs a;
+    a.P = W2;
+    a.Q = Hbuf;
+    a.O = Y;
+    a.ldp = ldw2;
+    a.ldq = FF;
+    a.ldo = ldy;
+    a.np = (int)D;
+    a.nq = (int)M;
+    a.k = (int)FF;
+    return finish(fsw::launch_stream_split(dtype, a, sp, ws2, (hipStream_t)stream));
+  }
   const size_t down_ws = (fsw_down_workspace_bytes(dtype, M, D, FF) + 255) & ~(size_t)255;
   rc = fsw_gateup_ws(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF, ws2 + down_ws,
                      fsw_gateup_workspace_bytes(dtype, M, 2 * FF, D), stream);

@@ -24,6 +24,10 @@ struct GemmArgs {
   // (gated kernel), bit 2 = P. A blocked [rows, k] matrix is ceil(rows / 256) panels of ceil(k / 32) blocks of
   // [256 rows][64 bytes], zero padded (blocked_bytes()).
   int layout = 0;
+  // words the FIRST workgroup of a gate/up launch sets to zero before anything else (tiled_dma_kernel and
+  // skinny_kernel honour it): the ticket counters of the split-K streaming down projection that follows in fsw_mlp
+  unsigned* zero_words = nullptr;
+  int n_zero_words = 0;
 };
 inline long long blocked_bytes(long long rows, long long k) {
   return ((rows + 255) / 256) * ((k + 31) / 32) * (256 * 64);
@@ -66,6 +70,17 @@ struct SkinnyPlan {
 };
 SkinnyPlan skinny_plan(bool gated, int np, int nq, int k);
 hipError_t launch_skinny(int dtype, bool gated, const GemmArgs& a, void* workspace, hipStream_t stream);
+
+// Split-K weight-streaming down projection for at most 32 activation rows (kernels_stream.hip): 32-row tiles, the K
+// range split over blockIdx.y, partial tiles reduced by the workgroup that draws a tile's last ticket.
+struct StreamPlan {
+  int splits;            // 0: the shape does not use this kernel
+  int tiles;
+  size_t partial_bytes;  // fp32 partial tiles, first in the scratch
+  int ticket_words;      // one counter per tile behind the partials; must be zero when the kernel starts
+};
+StreamPlan stream_split_plan(int np, int nq, int k, bool forced);  // forced: any supported shape
+hipError_t launch_stream_split(int dtype, const GemmArgs& a, const StreamPlan& p, void* workspace, hipStream_t stream);
 
 }  // namespace fsw
 

@@ -45,6 +45,8 @@ skinny_kernel(const GemmArgs a) {
   const int r16 = lane & 15;
   const int q = lane >> 4;
   const int p0 = blockIdx.x * R;     // first weight row of the tile (interleaved numbering when gated)
+  if (GATED && blockIdx.x == 0)      // counters of the kernel that follows in fsw_mlp (GemmArgs::zero_words)
+    for (int i = t; i < a.n_zero_words; i += NW * 64) a.zero_words[i] = 0u;
 
   const unsigned char* pbase = (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
   const __amdgpu_buffer_rsrc_t prs = make_rsrc(pbase, ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);

@@ -64,38 +64,6 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[FP][FQ], const GemmArgs
   }
 }
 
-// Gated epilogue that writes H panel-blocked for the down projection: panels of 256 activation rows, blocks of
-// 32 features, block (panel, j) = [256 rows][64 bytes] at ((panel * nblocks + j) * 256 + row) * 64. Every row of the
-// panel and every feature up to the next multiple of 32 is written: rows past nq and features past ff come from
-// out-of-range (zero) operand rows, so the padding the down projection's K loop reads is zero.
-template <class E, int WP, int WQ, int FP, int FQ>
-__device__ __forceinline__ void store_tile_blocked(f32x16 (&acc)[FP][FQ], const GemmArgs& a, int tp, int tq, int wp,
-                                                   int wq, int l32, int hi) {
-  constexpr int FO = FP / 2;
-  constexpr int BH = WP * FO;  // 32-feature blocks per tile
-  const int nblocks = (a.np / 2 + 31) >> 5;
-  unsigned char* O = (unsigned char*)a.O;
-#pragma unroll
-  for (int g = 0; g < FQ; ++g) {
-    const int row = (wq * FQ + g) * 32 + l32;
-#pragma unroll
-    for (int f = 0; f < FO; ++f) {
-      const int blk = tp * BH + wp * FO + f;
-      if (blk < nblocks) {
-        unsigned char* dst = O + (((long long)tq * nblocks + blk) * 256 + row) * 64 + hi * 8;
-#pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          float v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = acc[f][g][i4 * 4 + e] * silu_f32(acc[f + FO][g][i4 * 4 + e]);
-          u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
-          *(u32x2*)(dst + i4 * 16) = pk;
-        }
-      }
-    }
-  }
-}
-
 // Split-K epilogue of the plain kernel: fp32 partial sums to partial[split][m][n], 16 bytes per lane.
 template <int WP, int WQ, int FP, int FQ>
 __device__ __forceinline__ void store_partial(f32x16 (&acc)[FP][FQ], const GemmArgs& a, int split, int p0, int q0,
@@ -207,6 +175,8 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
   tile_coords(blockIdx.x, tiles_p, tiles_q, group, tp, tq);
   const int p0 = tp * BP;
   const int q0 = tq * BQ;
+  if (GATED && blockIdx.x == 0 && blockIdx.y == 0)  // counters of the kernel that follows in fsw_mlp (GemmArgs::zero_words)
+    for (int i = t; i < a.n_zero_words; i += NT) a.zero_words[i] = 0u;
 
   // ---- global -> LDS copy mapping: lane lands on chunk position pc of row rb (+ i * RSTEP)
   const int pc = t & 7;

@@ -20,7 +20,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 OBJ_DIR = os.path.join(HERE, "build", "hip_obj")
 LIB_NAME = "libfsw_hip.so"
-HIP_SOURCES = ["kernels_pair16.hip", "kernels_tiled.hip", "kernels_skinny.hip", "kernels_decode.hip", "probes.hip", "fsw_api.hip"]
+HIP_SOURCES = ["kernels_pair16.hip", "kernels_tiled.hip", "kernels_skinny.hip", "kernels_stream.hip", "kernels_decode.hip", "probes.hip", "fsw_api.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

@@ -178,7 +178,10 @@ FSW_API int fsw_version(void);
  * for M <= 64; the dispatcher itself picks it up to 16 .. 48 rows, the larger the weights the fewer); 102 is the
  * persistent streaming kernel (honoured for M <= 16; automatic only for d * ff >= 2^27); family 0 variant 101
  * makes fsw_mlp run M <= 16 as ONE persistent launch (gate/up, device-wide barrier, down) instead of two launches
- * -- see fsw_decode_barrier_failures(); 103 is 101 with a barrier that cannot complete (failure-path test).
+ * -- see fsw_decode_barrier_failures(); 103 is 101 with a barrier that cannot complete (failure-path test);
+ * family 1 variant 104 makes fsw_mlp run the down projection of M <= 32 rows on the split-K streaming kernel
+ * (32-row tiles, two K ranges whose partial tiles meet through ticket counters that the gate/up kernel zeroes)
+ * whatever the shape; the dispatcher picks it for 17 .. 32 rows of large weight matrices.
  * Returns FSW_E_VARIANT for unknown ids.
  */
 FSW_API int fsw_set_variant(int family, int variant);
@@ -207,7 +210,8 @@ FSW_API int fsw_probe_mfma(int dtype, int iters, const void* operands, void* out
 FSW_API int fsw_probe_read(const void* src, size_t bytes, void* out, int workgroups, void* stream);
 
 /* Name of the kernel variant the dispatcher picks for this shape (static storage); "splitk_<kernel>" when the
- * down projection splits K (family 1; K_or_FF decides). */
+ * down projection splits K (family 1; K_or_FF decides). family 2: the down projection as fsw_mlp runs it (differs
+ * from family 1, which is fsw_down on its own, for 17 .. 32 rows: "stream_split"). */
 FSW_API const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, int64_t K_or_FF);
 
 #ifdef __cplusplus

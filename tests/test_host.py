@@ -127,6 +127,11 @@ def test_variant_choice_by_regime(capi):
         assert name(1, 16, 8192, 28672) == "skinny"          # forced weight-streaming kernel wins over the size rule
         assert L.fsw_set_variant(1, 101) == capi.E_VARIANT   # the single-launch form is a family-0 (fsw_mlp) option
         assert L.fsw_set_variant(1, 103) == capi.E_VARIANT
+        assert L.fsw_set_variant(0, 104) == capi.E_VARIANT
+        # with the persistent streaming kernel forced for gate/up nothing zeroes the ticket counters: no split-K streaming
+        assert L.fsw_set_variant(1, 104) == capi.OK and capi.variant_name(2, 0, 4, 64, 32) == "skinny"
+        assert L.fsw_set_variant(0, -1) == capi.OK
+        assert capi.variant_name(2, 0, 4, 64, 32) == "stream_split" and name(1, 4, 64, 32) == "skinny"
     finally:
         L.fsw_set_variant(0, -1)
         L.fsw_set_variant(1, -1)

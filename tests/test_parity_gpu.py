@@ -263,6 +263,57 @@ def test_single_launch_decode_reports_a_failed_barrier(capi):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [1, 9, 16, 17, 32])
+def test_split_k_streaming_down_inside_mlp(capi, M, dtype):
+    """Inside fsw_mlp the down projection of up to 32 rows runs 32-row tiles with K split over two workgroups whose
+    partial tiles meet through ticket counters (zeroed by the gate/up kernel before it). Forced (variant 104) on small
+    and ragged shapes, automatic at decode size: against the oracle given the GPU's H, against the 16-row kernel, bit
+    for bit call after call (the summation order does not depend on which workgroup arrives last), and with a
+    workspace full of garbage (nothing but the gate/up kernel initialises the counters)."""
+    shapes = [(8, 8), (136, 40), (1000, 264), (520, 1032), (256, 2056), (40, 20000), (4096, 1032)]
+    for (d, ff) in shapes:
+        inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=53 * M + d, x_scale=0.5)
+        g = to_dev(inp)
+        try:
+            capi.set_variant(1, 104)
+            assert capi.variant_name(2, 0, M, d, ff) == "stream_split"
+            ws = capi.mlp_workspace(g["X"], ff)
+            ws.fill_(0xFF)
+            Y = capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws)
+            H = ws[: M * ff * 2].view(dtype).view(M, ff).clone()
+            reps = [capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws) for _ in range(5)]
+        finally:
+            capi.set_variant(1, -1)
+        assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype, "stream-split Y|H %s" % ((M, d, ff),))
+        oracle.assert_parity(Y, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64), "stream-split mlp %s" % ((M, d, ff),))
+        for r in reps:
+            assert torch.equal(r, Y)
+        try:
+            capi.set_variant(1, 100)
+            assert capi.variant_name(2, 0, M, d, ff) == "skinny"
+            Y16 = capi.mlp(g["X"], g["W13"], g["W2"])
+        finally:
+            capi.set_variant(1, -1)
+        assert (Y.float() - Y16.float()).abs().max().item() <= 2e-2
+    # automatic at decode size, and only there
+    name = lambda m, d_, ff_: capi.variant_name(2, 0, m, d_, ff_)
+    assert name(17, 4096, 14336) == "stream_split" and name(32, 4096, 14336) == "stream_split"
+    assert name(16, 4096, 14336) == "skinny" and name(24, 512, 1024) == "skinny" and name(33, 4096, 14336) != "stream_split"
+    assert name(16, 8192, 28672) == "decode_stream"
+    if M in (17, 32):
+        d, ff = 4096, 14336
+        inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=7, x_scale=0.5)
+        g = to_dev(inp)
+        ws = capi.mlp_workspace(g["X"], ff)
+        ws.fill_(0x5A)
+        Y = capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws)
+        H = ws[: M * ff * 2].view(dtype).view(M, ff).clone()
+        assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype, "stream-split decode size")
+        for _ in range(20):
+            assert torch.equal(capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws), Y)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_split_k_down_projection(capi, dtype):
     """65 <= M with few output tiles and a deep ff: fsw_down splits K across workgroups (fp32 partials in the
     workspace, then one rounding). Checked against the oracle and, bit for bit up to summation order, against the
