@@ -98,13 +98,15 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
                                     : (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
   const __amdgpu_buffer_rsrc_t prs =
       make_rsrc(pbase, PBLK ? (long long)nkt * PSTAGE : ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
-  unsigned poff[2 * LPH];
-#pragma unroll
-  for (int j = 0; j < 2 * LPH; ++j) {
-    const int r = rbp + j * 32;
-    const int grow = GATED ? (r < BP / 2 ? 2 * r : 2 * (r - BP / 2) + 1) : r;
-    poff[j] = (unsigned)grow * (unsigned)a.ldp * 2u + (unsigned)lcp * 16u;
-  }
+  // Copy instruction j of a pair covers LDS rows rbp + 32 j, i.e. weight rows (GATED: 2 rbp + 64 (j & 3) + (j >> 2),
+  // the even rows first, then the odd ones; else rbp + 32 j). Only the lane's part lives in a register; the part
+  // that depends on j and on the K position is wave-uniform and is added where the copy is issued (one VALU add per
+  // copy, in the shadow of the MFMAs): eight per-lane offsets held across the loop cost registers the accumulators
+  // need. The sum goes into the instruction's vector offset, which the hardware bounds-checks (rows past the matrix
+  // read as zero); its scalar offset is not checked.
+  const unsigned ldp2 = (unsigned)a.ldp * 2u;
+  const unsigned poff0 = (unsigned)(GATED ? 2 * rbp : rbp) * ldp2 + (unsigned)lcp * 16u;
+  auto p_row_off = [&](int j) -> unsigned { return (unsigned)(GATED ? 64 * (j & 3) + (j >> 2) : 32 * j) * ldp2; };
   // activation copy from the blocked panel: lane -> chunk position pcq of row rbq (+ 64 j)
   const int pcq = t & 3;
   const int rbq = t >> 2;
@@ -114,12 +116,23 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
                                     : (const unsigned char*)a.Q + (long long)tq * nkt * QSTAGE;
   const __amdgpu_buffer_rsrc_t qrs =
       make_rsrc(qbase, QROW ? ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2 : (long long)nkt * QSTAGE);
-  unsigned qoff[LQ];
-#pragma unroll
-  for (int j = 0; j < LQ; ++j)
-    qoff[j] = QROW ? (unsigned)(rbq + j * 64) * (unsigned)a.ldq * 2u + (unsigned)lcq * 16u
-                   : (unsigned)(rbq + j * 64) * 64u + (unsigned)lcq * 16u;
+  // Activation copy j covers rows rbq + 64 j. Blocked panels are zero padded and need no bounds check: the j and K
+  // parts go into the scalar offset. Row-major activations (QROW) are treated like the weights.
+  const unsigned ldq2 = (unsigned)a.ldq * 2u;
+  const unsigned qoff0 = QROW ? (unsigned)rbq * ldq2 + (unsigned)lcq * 16u : (unsigned)rbq * 64u + (unsigned)lcq * 16u;
   constexpr int QSTEP = QROW ? 64 : QSTAGE;  // bytes between consecutive K tiles of the activation operand
+  auto q_copy = [&](lds_void* dst, int j, int qt, bool qin) {
+    if constexpr (QROW) {
+      const unsigned voff = qoff0 + ((unsigned)(j * 64) * ldq2 + (unsigned)qt * 64u);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, dst, 16, (int)(qin ? voff : OOB_OFFSET), 0, 0, 0);
+    } else {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, dst, 16, (int)qoff0, j * 64 * 64 + qt * QSTAGE, 0, 0);
+    }
+  };
+  auto p_copy = [&](lds_void* dst, int j, int pair, bool in) {  // row-major weights: copy j (0 .. 7) of a K pair
+    const unsigned voff = poff0 + (p_row_off(j) + (unsigned)pair * 128u);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, dst, 16, (int)(in ? voff : OOB_OFFSET), 0, 0, 0);
+  };
 
   // operand fragment of a 16-row block: lane -> row r16, 16-byte K chunk c4 of the 32-element K tile
   const unsigned rd_p = PBLK ? (unsigned)((GATED ? wp * 64 : wp * 128) + r16) * 64u +
@@ -151,16 +164,14 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     const bool in = !KTAIL || (pair * 64 + lcp * 8) < a.k;
 #pragma unroll
     for (int i = LO; i < HI; ++i) {
-      if (i < LPH && PBLK) {  // weight tile kt + 3, copied like an activation tile
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + i * 64 * 64 + wave * 1024), 16, (int)qoff[i],
-                                                 qt * PSTAGE, 0, 0);
+      if (i < LPH && PBLK) {  // weight tile kt + 3, copied like a blocked activation tile (same lane mapping)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + i * 64 * 64 + wave * 1024), 16,
+                                                 (int)((unsigned)rbq * 64u + (unsigned)lcq * 16u), i * 64 * 64 + qt * PSTAGE, 0, 0);
       } else if (i < LPH) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + (half * LPH + i) * 32 * 128 + wave * 1024), 16,
-                                                 (int)(in ? poff[half * LPH + i] : OOB_OFFSET), pair * 128, 0, 0);
+        p_copy((lds_void*)(pslot + (half * LPH + i) * 32 * 128 + wave * 1024), half * LPH + i, pair, in);
       } else {
         const bool qin = !(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(qstage + (i - LPH) * 64 * 64 + wave * 1024), 16,
-                                                 (int)(qin ? qoff[i - LPH] : OOB_OFFSET), qt * QSTEP, 0, 0);
+        q_copy((lds_void*)(qstage + (i - LPH) * 64 * 64 + wave * 1024), i - LPH, qt, qin);
       }
     }
   };
@@ -170,24 +181,20 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     const bool in = !KTAIL || (pair * 64 + lcp * 8) < a.k;
 #pragma unroll
     for (int j = 0; j < 2 * LPH; ++j)
-      if (j >= j_lo && j < j_hi)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + j * 32 * 128 + wave * 1024), 16,
-                                                 (int)(in ? poff[j] : OOB_OFFSET), pair * 128, 0, 0);
+      if (j >= j_lo && j < j_hi) p_copy((lds_void*)(pslot + j * 32 * 128 + wave * 1024), j, pair, in);
   };
   auto dma_pb = [&](int pt_, unsigned char* pstage) {
     const int pt = pt_ < nkt ? pt_ : nkt - 1;
 #pragma unroll
     for (int j = 0; j < LPH; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pstage + j * 64 * 64 + wave * 1024), 16, (int)qoff[j],
-                                               pt * PSTAGE, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pstage + j * 64 * 64 + wave * 1024), 16,
+                                               (int)((unsigned)rbq * 64u + (unsigned)lcq * 16u), j * 64 * 64 + pt * PSTAGE, 0, 0);
   };
   auto dma_q = [&](int qt_, unsigned char* qstage) {
     const int qt = qt_ < nkt ? qt_ : nkt - 1;
     const bool qin = !(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k;
 #pragma unroll
-    for (int j = 0; j < LQ; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(qstage + j * 64 * 64 + wave * 1024), 16,
-                                               (int)(qin ? qoff[j] : OOB_OFFSET), qt * QSTEP, 0, 0);
+    for (int j = 0; j < LQ; ++j) q_copy((lds_void*)(qstage + j * 64 * 64 + wave * 1024), j, qt, qin);
   };
 
   // two register sets of the 16 fragments of a K tile: [0..7] weight blocks, [8..15] activation blocks
@@ -314,6 +321,11 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
 
   // epilogue: a lane owns activation row r16 of each block column and 4 consecutive features (4 c4 ..) per block row
   mfma_drain();
+  // The lane's coordinates are derived again here (from the hardware lane count, not from the values the loop set-up
+  // used): kept alive across the main loop they would not fit the register file beside the 256 accumulators and the
+  // two fragment sets, and the compiler would park them in scratch memory.
+  const int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  const int r16e = lane_e & 15, c4e = lane_e >> 4;
   if constexpr (OBLK) {
     // H panel-blocked (see store_tile_blocked): every row of the panel and every feature up to the next multiple
     // of 32 is written; padding comes out of zero operand rows
@@ -321,7 +333,7 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     unsigned char* O = (unsigned char*)a.O;
 #pragma unroll
     for (int g = 0; g < NB; ++g) {
-      const int row = wq * 128 + g * 16 + r16;
+      const int row = wq * 128 + g * 16 + r16e;
 #pragma unroll
       for (int f = 0; f < NB / 2; ++f) {
         const int blk = tp * 4 + wp * 2 + (f >> 1);
@@ -330,7 +342,7 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = acc[f][g][e] * silu_f32(acc[f + NB / 2][g][e]);
           u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
-          *(u32x2*)(O + (((long long)tq * nblocks + blk) * 256 + row) * 64 + (f & 1) * 32 + c4 * 8) = pk;
+          *(u32x2*)(O + (((long long)tq * nblocks + blk) * 256 + row) * 64 + (f & 1) * 32 + c4e * 8) = pk;
         }
       }
     }
@@ -339,12 +351,12 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     const bool vec_ok = (a.np & 3) == 0;
 #pragma unroll
     for (int g = 0; g < NB; ++g) {
-      const int m = q0 + wq * 128 + g * 16 + r16;
+      const int m = q0 + wq * 128 + g * 16 + r16e;
       if (m >= a.nq) continue;
       float* prow = part + (long long)m * a.np;
 #pragma unroll
       for (int f = 0; f < NB; ++f) {
-        const int n = p0 + wp * 128 + f * 16 + c4 * 4;
+        const int n = p0 + wp * 128 + f * 16 + c4e * 4;
         if (vec_ok && n + 3 < a.np) {
           *(f32x4*)(prow + n) = acc[f][g];
         } else {
@@ -361,12 +373,12 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     const bool vec_ok = ((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 7) == 0);
 #pragma unroll
     for (int g = 0; g < NB; ++g) {
-      const int m = q0 + wq * 128 + g * 16 + r16;
+      const int m = q0 + wq * 128 + g * 16 + r16e;
       if (m >= a.nq) continue;
       unsigned short* orow = O + (long long)m * a.ldo;
 #pragma unroll
       for (int f = 0; f < FO; ++f) {
-        const int n = (GATED ? p0 / 2 + wp * 64 : p0 + wp * 128) + f * 16 + c4 * 4;
+        const int n = (GATED ? p0 / 2 + wp * 64 : p0 + wp * 128) + f * 16 + c4e * 4;
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = GATED ? acc[f][g][e] * silu_f32(acc[f + FO][g][e]) : acc[f][g][e];
