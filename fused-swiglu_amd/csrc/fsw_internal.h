@@ -44,7 +44,7 @@ int pair16_variant();  // index of the 256 x 256 kernel in the table
 const TiledVariant& tiled_variant(int variant);
 // row-major operands (GemmArgs::layout 0)
 hipError_t launch_tiled(int variant, int dtype, bool gated, const GemmArgs& a, hipStream_t stream);
-int raster_group(bool gated);  // activation-row tiles per raster band of the tiled kernels
+int raster_group(bool gated, int tiles_q);  // activation-row tiles per raster band of the tiled kernels
 // The 256 x 256 kernel on v_mfma_f32_16x16x32 (kernels_pair16.hip) for GemmArgs::layout 0, 1, 3, 5, 7.
 // gated: X blocked in (bit 0), H blocked out (bit 1) or row-major, W13 blocked (bit 2) or row-major: layouts 1, 3, 5, 7;
 // plain: H blocked in, W2 row-major (1) or blocked (5); 0 = everything row-major

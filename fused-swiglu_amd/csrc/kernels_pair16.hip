@@ -20,12 +20,13 @@ typedef __attribute__((address_space(3))) void lds_void;
 // between MFMAs), and the MFMA is written out with its destination tied to the addend (mfma16_acc).
 //
 // Operands go global -> LDS with buffer_load ... lds. The activation operand is panel-blocked (blocks of
-// [256 rows][32 elements], 16 KB contiguous) and keeps a ring of four 16 KB stages; a tile is issued three iterations
-// before it is multiplied. The weight operand is ROW-MAJOR: read 32 K elements at a time it would yield 64-byte
-// requests, half a cache line each, so it is fetched in K PAIRS (64 elements = one 128-byte line per row) into a ring
-// of three 32 KB pair slots, half a pair per iteration, four to three iterations ahead. The slot/stage pattern
-// repeats every 12 K tiles (lcm of 6 and 4): the loop is unrolled twelvefold with every LDS address a compile-time
-// constant. 160 KB of LDS.
+// [256 rows][32 elements], 16 KB contiguous) and keeps four 16 KB stages = two K pairs. The weight operand is
+// ROW-MAJOR: read 32 K elements at a time it would yield 64-byte requests, half a cache line each, so it is fetched in
+// K PAIRS (64 elements = one 128-byte line per row) into a ring of three 32 KB pair slots. 160 KB of LDS.
+// The main loop walks K in pairs with ONE workgroup barrier per pair (see pair_iteration); the slot/stage pattern
+// repeats every 6 pairs (lcm of 3 and 2), so the loop is unrolled sixfold with every LDS address a compile-time
+// constant. Measured against one barrier per K tile (copies three tiles ahead): gate/up 1.285 -> 1.270 ms at
+// 8192 x 4096 x 28672, bit-identical results (the K order is the same).
 // LDS layouts: pair slot = [256 rows][128 B], chunk c of row r at position c ^ ((r >> 1) & 7); activation stage =
 // [256 rows][64 B], chunk c at c ^ ((r >> 2) & 3): the 16 rows a fragment read touches at one logical chunk cover
 // the 64 banks once. The swizzle is applied on the global side of the copy (which lane fetches which chunk), since
@@ -58,7 +59,6 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   constexpr int PSLOT = BP * 128, QSTAGE = BQ * 64;
   constexpr int LPH = 4;  // weight copy instructions per wave per HALF pair (8 rows x 128 B each)
   constexpr int LQ = 4;   // activation copy instructions per wave per K tile (16 rows x 64 B each)
-  constexpr int NL = LPH + LQ;
   static_assert(!OBLK || GATED, "only H is ever written blocked");
   static_assert(!PBLK || !KTAIL, "blocked operands are zero padded in K");
   constexpr int PSTAGE = BP * 64;
@@ -120,15 +120,6 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   // parts go into the scalar offset. Row-major activations (QROW) are treated like the weights.
   const unsigned ldq2 = (unsigned)a.ldq * 2u;
   const unsigned qoff0 = QROW ? (unsigned)rbq * ldq2 + (unsigned)lcq * 16u : (unsigned)rbq * 64u + (unsigned)lcq * 16u;
-  constexpr int QSTEP = QROW ? 64 : QSTAGE;  // bytes between consecutive K tiles of the activation operand
-  auto q_copy = [&](lds_void* dst, int j, int qt, bool qin) {
-    if constexpr (QROW) {
-      const unsigned voff = qoff0 + ((unsigned)(j * 64) * ldq2 + (unsigned)qt * 64u);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, dst, 16, (int)(qin ? voff : OOB_OFFSET), 0, 0, 0);
-    } else {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, dst, 16, (int)qoff0, j * 64 * 64 + qt * QSTAGE, 0, 0);
-    }
-  };
   auto p_copy = [&](lds_void* dst, int j, int pair, bool in) {  // row-major weights: copy j (0 .. 7) of a K pair
     const unsigned voff = poff0 + (p_row_off(j) + (unsigned)pair * 128u);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, dst, 16, (int)(in ? voff : OOB_OFFSET), 0, 0, 0);
@@ -154,62 +145,19 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
 #pragma unroll
     for (int g = 0; g < NB; ++g) acc[f][g] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // copy instruction idx of iteration kt: 0..3 = half (kt & 1) of weight pair (kt >> 1) + 2, 4..7 = activation tile
-  // kt + 3. Past the end both re-read the last pair / tile (never consumed).
-  auto dma = [&](int kt, unsigned char* pslot, unsigned char* qstage, auto lo_c, auto hi_c) {
-    constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
-    const int pair = (kt >> 1) + 2 < npair ? (kt >> 1) + 2 : npair - 1;
-    const int half = kt & 1;
-    const int qt = kt + 3 < nkt ? kt + 3 : nkt - 1;
-    const bool in = !KTAIL || (pair * 64 + lcp * 8) < a.k;
-#pragma unroll
-    for (int i = LO; i < HI; ++i) {
-      if (i < LPH && PBLK) {  // weight tile kt + 3, copied like a blocked activation tile (same lane mapping)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pslot + i * 64 * 64 + wave * 1024), 16,
-                                                 (int)((unsigned)rbq * 64u + (unsigned)lcq * 16u), i * 64 * 64 + qt * PSTAGE, 0, 0);
-      } else if (i < LPH) {
-        p_copy((lds_void*)(pslot + (half * LPH + i) * 32 * 128 + wave * 1024), half * LPH + i, pair, in);
-      } else {
-        const bool qin = !(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k;
-        q_copy((lds_void*)(qstage + (i - LPH) * 64 * 64 + wave * 1024), i - LPH, qt, qin);
-      }
-    }
-  };
-  // prologue copies: a whole weight pair / one activation tile
-  auto dma_pair = [&](int pair_, unsigned char* pslot, int j_lo, int j_hi) {
-    const int pair = pair_ < npair ? pair_ : npair - 1;
-    const bool in = !KTAIL || (pair * 64 + lcp * 8) < a.k;
-#pragma unroll
-    for (int j = 0; j < 2 * LPH; ++j)
-      if (j >= j_lo && j < j_hi) p_copy((lds_void*)(pslot + j * 32 * 128 + wave * 1024), j, pair, in);
-  };
-  auto dma_pb = [&](int pt_, unsigned char* pstage) {
-    const int pt = pt_ < nkt ? pt_ : nkt - 1;
-#pragma unroll
-    for (int j = 0; j < LPH; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(pstage + j * 64 * 64 + wave * 1024), 16,
-                                               (int)((unsigned)rbq * 64u + (unsigned)lcq * 16u), j * 64 * 64 + pt * PSTAGE, 0, 0);
-  };
-  auto dma_q = [&](int qt_, unsigned char* qstage) {
-    const int qt = qt_ < nkt ? qt_ : nkt - 1;
-    const bool qin = !(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k;
-#pragma unroll
-    for (int j = 0; j < LQ; ++j) q_copy((lds_void*)(qstage + j * 64 * 64 + wave * 1024), j, qt, qin);
-  };
-
   // two register sets of the 16 fragments of a K tile: [0..7] weight blocks, [8..15] activation blocks
   u32x4 fr[2][2 * NB];
-  using C0 = std::integral_constant<int, 0>;
-  using CH = std::integral_constant<int, LPH>;
-  // The barrier sits in the middle of the iteration. At the barrier of iteration kt everything issued up to
-  // iteration kt - 2 has landed (tile kt + 1 and its weight pair among it); the copies of iteration kt - 1 and of
-  // this one stay in flight. lgkmcnt(0): this wave's reads of tile kt (issued in the second half of
-  // iteration kt - 1) are complete, so its stage may be refilled from the next iteration on.
-  constexpr int VM = NL + NL;
+  // ONE workgroup barrier per K PAIR (two K tiles, 128 MFMAs per wave). Pair iteration I works on tile a = 2I (fragments
+  // in register set 0) and tile b = 2I + 1 (set 1) in four quarters of 32 MFMAs:
+  //   Q1  a, weight blocks 0..3   + the 8 activation copies of pair I + 1 (its two stages were freed by barrier I - 1)
+  //   Q2  a, weight blocks 4..7   + the 16 fragment reads of b
+  //   Q3  b, weight blocks 0..3   + the 8 weight copies of pair I + 2 (into the slot of pair I - 1)
+  //   barrier: everything but the 8 copies of Q3 has landed (pair I + 1 complete); every wave has read a and b
+  //   Q4  b, weight blocks 4..7   + the 16 fragment reads of tile a of pair I + 1
+  // Prepacked weights (PBLK) have two double stages like the activations: their 8 copies of pair I + 1 go into Q1 as
+  // well and nothing stays in flight at the barrier.
+  constexpr int VM = PBLK ? 0 : 2 * LPH;
   constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
-
-  // Fragment read by index: weight block 0, the 8 activation blocks, then weight blocks 1 .. 7: the order the MFMAs
-  // (f major, g minor) first need them.
   auto read_one = [&](int set, int idx, const unsigned char* pslot, int half, const unsigned char* qstage) {
     if (idx == 0) {
       fr[set][0] = *(const u32x4*)(pslot + rd_p + p_block_off(0) + (PBLK ? 0u : xp[half]));
@@ -222,101 +170,127 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   auto mma_one = [&](int set, int i) {
     E::mfma16_acc(acc[i / NB][i % NB], fr[set][i / NB], fr[set][NB + i % NB]);
   };
-  // iteration j (mod 12) of the unrolled loop, K tile kt = base + j, fragments of tile kt in register set j & 1.
-  // First half: the 32 MFMAs of weight blocks 0 .. 3 with the eight copies between them (one per four MFMAs);
-  // barrier; second half: the 32 MFMAs of weight blocks 4 .. 7 with the 16 fragment reads of tile kt + 1 (one per two
-  // MFMAs). The scheduler is fenced after every group, so this is the issue order. (A copy next to a read between two
-  // 16-cycle MFMAs — s_mov m0, the copy, the read, a wait — does not fit their shadow.)
-  auto iteration = [&](auto j_c, int kt) {
-    constexpr int J = decltype(j_c)::value;
-    constexpr int SET = J & 1;
-    unsigned char* const p_nxt = PBLK ? ps[(J + 1) & 3] : ps[((J + 1) >> 1) % 3];
-    unsigned char* const p_fill = PBLK ? ps[(J + 3) & 3] : ps[((J >> 1) + 2) % 3];
-    unsigned char* const q_nxt = qs[(J + 1) & 3];
-    unsigned char* const q_fill = qs[(J + 3) & 3];
-#define FSW_P16_GROUP(G)                                                                                      \
-    mma_one(SET, 8 * (G) + 0);                                                                                 \
-    mma_one(SET, 8 * (G) + 1);                                                                                 \
-    dma(kt, p_fill, q_fill, std::integral_constant<int, 2 * (G)>{}, std::integral_constant<int, 2 * (G) + 1>{}); \
-    __builtin_amdgcn_sched_barrier(0);                                                                         \
-    mma_one(SET, 8 * (G) + 2);                                                                                 \
-    mma_one(SET, 8 * (G) + 3);                                                                                 \
-    mma_one(SET, 8 * (G) + 4);                                                                                 \
-    mma_one(SET, 8 * (G) + 5);                                                                                 \
-    dma(kt, p_fill, q_fill, std::integral_constant<int, 2 * (G) + 1>{}, std::integral_constant<int, 2 * (G) + 2>{}); \
-    __builtin_amdgcn_sched_barrier(0);                                                                         \
-    mma_one(SET, 8 * (G) + 6);                                                                                 \
-    mma_one(SET, 8 * (G) + 7);                                                                                 \
-    __builtin_amdgcn_sched_barrier(0);
-    FSW_P16_GROUP(0)
-    FSW_P16_GROUP(1)
-    FSW_P16_GROUP(2)
-    FSW_P16_GROUP(3)
-#undef FSW_P16_GROUP
-    asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(WAIT_IMM) : "memory");
+  // activation copy j (0 .. 7) of pair `pair`: tile 2 pair + j / 4; tiles past the end arrive as zeros
+  auto q_pair_copy = [&](unsigned char* st_a, unsigned char* st_b, int pair, int j) {
+    const int qt = 2 * pair + j / LQ;
+    unsigned char* st = j < LQ ? st_a : st_b;
+    lds_void* dst = (lds_void*)(st + (j % LQ) * 64 * 64 + wave * 1024);
+    const bool qin = qt < nkt && (!(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k);
+    if constexpr (QROW) {
+      const unsigned voff = qoff0 + ((unsigned)((j % LQ) * 64) * ldq2 + (unsigned)qt * 64u);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, dst, 16, (int)(qin ? voff : OOB_OFFSET), 0, 0, 0);
+    } else {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, dst, 16, (int)(qin ? qoff0 : OOB_OFFSET), (j % LQ) * 64 * 64 + qt * QSTAGE, 0,
+                                               0);
+    }
+  };
+  // weight copy j (0 .. 7) of pair `pair`: row-major: rows of the pair slot; prepacked: tile 2 pair + j / 4
+  auto p_pair_copy = [&](unsigned char* st_a, unsigned char* st_b, int pair, int j) {
+    if constexpr (PBLK) {
+      const int pt = 2 * pair + j / LPH;
+      unsigned char* st = j < LPH ? st_a : st_b;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(st + (j % LPH) * 64 * 64 + wave * 1024), 16,
+                                               (int)(pt < nkt ? (unsigned)rbq * 64u + (unsigned)lcq * 16u : OOB_OFFSET),
+                                               (j % LPH) * 64 * 64 + pt * PSTAGE, 0, 0);
+    } else {
+      const int pc = pair < npair ? pair : npair - 1;  // past the end: re-read the last pair, never multiplied
+      const bool in = !KTAIL || (pc * 64 + lcp * 8) < a.k;
+      p_copy((lds_void*)(st_a + j * 32 * 128 + wave * 1024), j, pc, in);
+    }
+  };
+  auto pair_iteration = [&](auto i_c, int pr) {
+    constexpr int I = decltype(i_c)::value;  // pair index modulo 6: LDS addresses are compile-time constants
+    unsigned char* const pa = PBLK ? ps[(2 * I) & 3] : ps[I % 3];
+    unsigned char* const pb = PBLK ? ps[(2 * I + 1) & 3] : ps[I % 3];
+    unsigned char* const pna = PBLK ? ps[(2 * I + 2) & 3] : ps[(I + 1) % 3];
+    unsigned char* const pnb = PBLK ? ps[(2 * I + 3) & 3] : ps[(I + 1) % 3];
+    unsigned char* const pfill = PBLK ? pna : ps[(I + 2) % 3];
+    unsigned char* const qa = qs[(2 * I) & 3];
+    unsigned char* const qb = qs[(2 * I + 1) & 3];
+    unsigned char* const qna = qs[(2 * I + 2) & 3];
+    unsigned char* const qnb = qs[(2 * I + 3) & 3];
+    (void)pa; (void)qa; (void)pnb; (void)qnb; (void)pfill;
+    // Q1
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      mma_one(0, 4 * c + 0);
+      mma_one(0, 4 * c + 1);
+      q_pair_copy(qna, qnb, pr + 1, c);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_one(0, 4 * c + 2);
+      if constexpr (PBLK) {
+        p_pair_copy(pna, pnb, pr + 1, c);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mma_one(0, 4 * c + 3);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // Q2
 #pragma unroll
     for (int r = 0; r < 2 * NB; ++r) {
-      mma_one(SET, 4 * NB + 2 * r);
-      read_one(SET ^ 1, r, p_nxt, (J + 1) & 1, q_nxt);
-      mma_one(SET, 4 * NB + 2 * r + 1);
+      mma_one(0, 4 * NB + 2 * r);
+      read_one(1, r, pb, 1, qb);
+      mma_one(0, 4 * NB + 2 * r + 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // Q3
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      mma_one(1, 4 * c + 0);
+      mma_one(1, 4 * c + 1);
+      if constexpr (!PBLK) {
+        p_pair_copy(pfill, pfill, pr + 2, c);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mma_one(1, 4 * c + 2);
+      mma_one(1, 4 * c + 3);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(WAIT_IMM) : "memory");
+    // Q4
+#pragma unroll
+    for (int r = 0; r < 2 * NB; ++r) {
+      mma_one(1, 4 * NB + 2 * r);
+      read_one(0, r, pna, 0, qna);
+      mma_one(1, 4 * NB + 2 * r + 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
 
   if (nkt > 0) {
-    // fill in the order the loop would have issued it: [pair 0, tile 0] [pair 1 first half, tile 1] [pair 1 second
-    // half, tile 2]; then pair 0 and tile 0 have landed when 16 copies are still in flight
-    if constexpr (PBLK) {
-      dma_pb(0, ps0);
-      dma_q(0, qs0);
-      dma_pb(1, ps1);
-      dma_q(1, qs1);
-      dma_pb(2, ps2);
-      dma_q(2, qs2);
-    } else {
-      dma_pair(0, ps0, 0, 2 * LPH);
-      dma_q(0, qs0);
-      dma_pair(1, ps1, 0, LPH);
-      dma_q(1, qs1);
-      dma_pair(1, ps1, LPH, 2 * LPH);
-      dma_q(2, qs2);
+    // weight pairs 0 and 1, activation pair 0; pair 0 has landed when the 8 copies of weight pair 1 are still in flight
+#pragma unroll
+    for (int j = 0; j < 8; ++j) p_pair_copy(ps0, PBLK ? ps1 : ps0, 0, j);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) q_pair_copy(qs0, qs1, 0, j);
+    if constexpr (!PBLK) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) p_pair_copy(ps1, ps1, 1, j);
     }
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NL) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(VM) : "memory");
 #pragma unroll
     for (int i = 0; i < 2 * NB; ++i) read_one(0, i, ps0, 0, qs0);
   }
-  int kt = 0;
-  for (; kt + 11 < nkt; kt += 12) {
-    iteration(std::integral_constant<int, 0>{}, kt);
-    iteration(std::integral_constant<int, 1>{}, kt + 1);
-    iteration(std::integral_constant<int, 2>{}, kt + 2);
-    iteration(std::integral_constant<int, 3>{}, kt + 3);
-    iteration(std::integral_constant<int, 4>{}, kt + 4);
-    iteration(std::integral_constant<int, 5>{}, kt + 5);
-    iteration(std::integral_constant<int, 6>{}, kt + 6);
-    iteration(std::integral_constant<int, 7>{}, kt + 7);
-    iteration(std::integral_constant<int, 8>{}, kt + 8);
-    iteration(std::integral_constant<int, 9>{}, kt + 9);
-    iteration(std::integral_constant<int, 10>{}, kt + 10);
-    iteration(std::integral_constant<int, 11>{}, kt + 11);
+  int pr = 0;
+  for (; pr + 5 < npair; pr += 6) {
+    pair_iteration(std::integral_constant<int, 0>{}, pr);
+    pair_iteration(std::integral_constant<int, 1>{}, pr + 1);
+    pair_iteration(std::integral_constant<int, 2>{}, pr + 2);
+    pair_iteration(std::integral_constant<int, 3>{}, pr + 3);
+    pair_iteration(std::integral_constant<int, 4>{}, pr + 4);
+    pair_iteration(std::integral_constant<int, 5>{}, pr + 5);
   }
-#define FSW_PAIR16_TAIL(J)                                     \
-  if (kt < nkt) {                                            \
-    iteration(std::integral_constant<int, J>{}, kt);         \
-    ++kt;                                                    \
+#define FSW_PAIR16_TAIL(I)                                        \
+  if (pr < npair) {                                             \
+    pair_iteration(std::integral_constant<int, I>{}, pr);      \
+    ++pr;                                                       \
   }
   FSW_PAIR16_TAIL(0)
   FSW_PAIR16_TAIL(1)
   FSW_PAIR16_TAIL(2)
   FSW_PAIR16_TAIL(3)
   FSW_PAIR16_TAIL(4)
-  FSW_PAIR16_TAIL(5)
-  FSW_PAIR16_TAIL(6)
-  FSW_PAIR16_TAIL(7)
-  FSW_PAIR16_TAIL(8)
-  FSW_PAIR16_TAIL(9)
-  FSW_PAIR16_TAIL(10)
 #undef FSW_PAIR16_TAIL
 
   // epilogue: a lane owns activation row r16 of each block column and 4 consecutive features (4 c4 ..) per block row
@@ -406,10 +380,10 @@ hipError_t launch_pair16_blocked_x(const GemmArgs& a, hipStream_t stream) {
   const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
   if (a.k % 64 == 0) {
     hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK>), grid, block, 0, stream, a, tiles_p, tiles_q,
-                       raster_group(GATED));
+                       raster_group(GATED, tiles_q));
   } else {
     hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, OBLK>), grid, block, 0, stream, a, tiles_p, tiles_q,
-                       raster_group(GATED));
+                       raster_group(GATED, tiles_q));
   }
   return hipGetLastError();
 }
@@ -423,10 +397,10 @@ hipError_t launch_pair16_rowmajor(const GemmArgs& a, hipStream_t stream) {
   const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
   if (a.k % 64 == 0) {
     hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, false, false, true>), grid, block, 0, stream, a, tiles_p,
-                       tiles_q, raster_group(GATED));
+                       tiles_q, raster_group(GATED, tiles_q));
   } else {
     hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, false, false, true>), grid, block, 0, stream, a, tiles_p,
-                       tiles_q, raster_group(GATED));
+                       tiles_q, raster_group(GATED, tiles_q));
   }
   return hipGetLastError();
 }
@@ -440,10 +414,10 @@ hipError_t launch_pair16_split(const GemmArgs& a, hipStream_t stream) {
   const dim3 grid((unsigned)(tiles_p * tiles_q), (unsigned)a.splits), block(256);
   if (a.k % 64 == 0) {
     hipLaunchKernelGGL((tiled_pair16_kernel<E, false, false, false, false, true, true>), grid, block, 0, stream, a,
-                       tiles_p, tiles_q, raster_group(false));
+                       tiles_p, tiles_q, raster_group(false, tiles_q));
   } else {
     hipLaunchKernelGGL((tiled_pair16_kernel<E, false, true, false, false, true, true>), grid, block, 0, stream, a,
-                       tiles_p, tiles_q, raster_group(false));
+                       tiles_p, tiles_q, raster_group(false, tiles_q));
   }
   return hipGetLastError();
 }
@@ -455,7 +429,7 @@ hipError_t launch_pair16_blocked_xw(const GemmArgs& a, hipStream_t stream) {
   const int tiles_q = (a.nq + 255) / 256;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
   hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK, true>), dim3((unsigned)(tiles_p * tiles_q)), dim3(256), 0,
-                     stream, a, tiles_p, tiles_q, raster_group(GATED));
+                     stream, a, tiles_p, tiles_q, raster_group(GATED, tiles_q));
   return hipGetLastError();
 }
 

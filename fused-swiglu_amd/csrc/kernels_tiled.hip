@@ -445,9 +445,12 @@ constexpr int kPair16Variant = 5;
 
 }  // namespace
 
-// Activation-row tiles per raster band. Measured on the headline shapes: the gate/up product (many weight
-// panels, 4096-deep K) prefers 4, the down product (few weight panels, 14336-deep K) prefers 2.
-int raster_group(bool gated) { return gated ? 4 : 2; }
+// Activation-row tiles per raster band of the 256 x 256 kernel (the 128-row kernels above use 4 for the gate/up and
+// 2 for the down product): 4, i.e. the 32 tiles an XCD runs at once are 4 activation panels x 8 weight
+// panels (12 operand panels through its L2 per round). The down product of tall problems (32 activation tiles or
+// more, 16 weight panels, 14336-deep K) measures level to 1 % slower that way and keeps bands of 2; with fewer
+// activation tiles bands of 4 win (4096 x 4096 x 11008: 244 -> 236 us, 2048 x 8192 x 28672 fp16: 639 -> 633 us).
+int raster_group(bool gated, int tiles_q) { return gated ? 4 : (tiles_q >= 32 ? 2 : 4); }
 
 namespace {
 
@@ -479,9 +482,9 @@ hipError_t launch_dma(const GemmArgs& a, hipStream_t stream) {
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
   const dim3 grid((unsigned)(tiles_p * tiles_q));
   if (a.k % 64 == 0) {
-    launch_dma_kernel<E, GATED, false, WP, WQ, FP, FQ>(grid, stream, a, tiles_p, tiles_q, raster_group(GATED));
+    launch_dma_kernel<E, GATED, false, WP, WQ, FP, FQ>(grid, stream, a, tiles_p, tiles_q, GATED ? 4 : 2);
   } else {
-    launch_dma_kernel<E, GATED, true, WP, WQ, FP, FQ>(grid, stream, a, tiles_p, tiles_q, raster_group(GATED));
+    launch_dma_kernel<E, GATED, true, WP, WQ, FP, FQ>(grid, stream, a, tiles_p, tiles_q, GATED ? 4 : 2);
   }
   return hipGetLastError();
 }
@@ -610,7 +613,7 @@ hipError_t launch_splitk_one(const GemmArgs& a, hipStream_t stream) {
   const int tiles_q = (a.nq + BQ - 1) / BQ;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
   const dim3 grid((unsigned)(tiles_p * tiles_q), (unsigned)a.splits);
-  const int group = raster_group(false);
+  const int group = 2;
   if (a.k % 64 == 0) {
     launch_dma_kernel<E, false, false, WP, WQ, FP, FQ>(grid, stream, a, tiles_p, tiles_q, group);
   } else {
