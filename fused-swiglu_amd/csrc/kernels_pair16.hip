@@ -34,8 +34,8 @@ typedef __attribute__((address_space(3))) void lds_void;
 // to LDS rows 0..127 and the odd ("gate") rows to 128..255; a wave multiplies 64 of each against the same activation
 // fragments, so up and gate of one output land in the same lane and register index.
 // PBLK: the weight operand is panel-blocked as well (prepacked; for the gated kernel in de-interleaved row order). It
-// then arrives like the activations, one 16 KB block per K tile, and keeps a ring of four 64-byte-row stages instead
-// of the pair slots (128 KB of LDS).
+// then arrives like the activations, one 16 KB block per K tile; a pair slot holds the two blocks of a K pair, one
+// after the other, as 64-byte rows, and the ring of three slots runs on the same schedule as for row-major weights.
 // QROW: the activation operand is row-major (callers without scratch for a blocked copy; few ragged activation
 // panels, where re-blocking does not pay): 64-byte requests per row and K tile, rows past nq read as zero.
 // SPLIT (row-major operands, plain product): blockIdx.y selects one of a.splits contiguous runs of 64-element K
@@ -62,17 +62,15 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   static_assert(!OBLK || GATED, "only H is ever written blocked");
   static_assert(!PBLK || !KTAIL, "blocked operands are zero padded in K");
   constexpr int PSTAGE = BP * 64;
-  constexpr int PBUF = PBLK ? PSTAGE : PSLOT;
 
-  __shared__ __align__(1024) unsigned char ps0[PBUF];
-  __shared__ __align__(1024) unsigned char ps1[PBUF];
-  __shared__ __align__(1024) unsigned char ps2[PBUF];
-  __shared__ alignas(PBLK ? 1024 : 16) unsigned char ps3[PBLK ? PSTAGE : 16];
+  __shared__ __align__(1024) unsigned char ps0[PSLOT];
+  __shared__ __align__(1024) unsigned char ps1[PSLOT];
+  __shared__ __align__(1024) unsigned char ps2[PSLOT];
   __shared__ __align__(1024) unsigned char qs0[QSTAGE];
   __shared__ __align__(1024) unsigned char qs1[QSTAGE];
   __shared__ __align__(1024) unsigned char qs2[QSTAGE];
   __shared__ __align__(1024) unsigned char qs3[QSTAGE];
-  unsigned char* const ps[4] = {ps0, ps1, ps2, ps3};
+  unsigned char* const ps[3] = {ps0, ps1, ps2};
   unsigned char* const qs[4] = {qs0, qs1, qs2, qs3};
 
   const int t = threadIdx.x;
@@ -154,9 +152,7 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   //   Q3  b, weight blocks 0..3   + the 8 weight copies of pair I + 2 (into the slot of pair I - 1)
   //   barrier: everything but the 8 copies of Q3 has landed (pair I + 1 complete); every wave has read a and b
   //   Q4  b, weight blocks 4..7   + the 16 fragment reads of tile a of pair I + 1
-  // Prepacked weights (PBLK) have two double stages like the activations: their 8 copies of pair I + 1 go into Q1 as
-  // well and nothing stays in flight at the barrier.
-  constexpr int VM = PBLK ? 0 : 2 * LPH;
+  constexpr int VM = 2 * LPH;
   constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
   auto read_one = [&](int set, int idx, const unsigned char* pslot, int half, const unsigned char* qstage) {
     if (idx == 0) {
@@ -184,32 +180,31 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
                                                0);
     }
   };
-  // weight copy j (0 .. 7) of pair `pair`: row-major: rows of the pair slot; prepacked: tile 2 pair + j / 4
-  auto p_pair_copy = [&](unsigned char* st_a, unsigned char* st_b, int pair, int j) {
+  // weight copy j (0 .. 7) of pair `pair` into a pair slot: row-major: 32 rows of 128 bytes; prepacked: a quarter of
+  // the block of K tile 2 pair + j / 4 (the second block of the pair sits PSTAGE bytes into the slot)
+  auto p_pair_copy = [&](unsigned char* slot, int pair, int j) {
     if constexpr (PBLK) {
       const int pt = 2 * pair + j / LPH;
-      unsigned char* st = j < LPH ? st_a : st_b;
+      unsigned char* st = slot + (j / LPH) * PSTAGE;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, (lds_void*)(st + (j % LPH) * 64 * 64 + wave * 1024), 16,
                                                (int)(pt < nkt ? (unsigned)rbq * 64u + (unsigned)lcq * 16u : OOB_OFFSET),
                                                (j % LPH) * 64 * 64 + pt * PSTAGE, 0, 0);
     } else {
       const int pc = pair < npair ? pair : npair - 1;  // past the end: re-read the last pair, never multiplied
       const bool in = !KTAIL || (pc * 64 + lcp * 8) < a.k;
-      p_copy((lds_void*)(st_a + j * 32 * 128 + wave * 1024), j, pc, in);
+      p_copy((lds_void*)(slot + j * 32 * 128 + wave * 1024), j, pc, in);
     }
   };
   auto pair_iteration = [&](auto i_c, int pr) {
     constexpr int I = decltype(i_c)::value;  // pair index modulo 6: LDS addresses are compile-time constants
-    unsigned char* const pa = PBLK ? ps[(2 * I) & 3] : ps[I % 3];
-    unsigned char* const pb = PBLK ? ps[(2 * I + 1) & 3] : ps[I % 3];
-    unsigned char* const pna = PBLK ? ps[(2 * I + 2) & 3] : ps[(I + 1) % 3];
-    unsigned char* const pnb = PBLK ? ps[(2 * I + 3) & 3] : ps[(I + 1) % 3];
-    unsigned char* const pfill = PBLK ? pna : ps[(I + 2) % 3];
+    unsigned char* const pb = ps[I % 3] + (PBLK ? PSTAGE : 0);  // tile b of this pair
+    unsigned char* const pna = ps[(I + 1) % 3];                 // tile a of the next pair
+    unsigned char* const pfill = ps[(I + 2) % 3];
     unsigned char* const qa = qs[(2 * I) & 3];
     unsigned char* const qb = qs[(2 * I + 1) & 3];
     unsigned char* const qna = qs[(2 * I + 2) & 3];
     unsigned char* const qnb = qs[(2 * I + 3) & 3];
-    (void)pa; (void)qa; (void)pnb; (void)qnb; (void)pfill;
+    (void)qa;
     // Q1
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
@@ -218,10 +213,6 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
       q_pair_copy(qna, qnb, pr + 1, c);
       __builtin_amdgcn_sched_barrier(0);
       mma_one(0, 4 * c + 2);
-      if constexpr (PBLK) {
-        p_pair_copy(pna, pnb, pr + 1, c);
-        __builtin_amdgcn_sched_barrier(0);
-      }
       mma_one(0, 4 * c + 3);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -238,10 +229,8 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     for (int c = 0; c < 8; ++c) {
       mma_one(1, 4 * c + 0);
       mma_one(1, 4 * c + 1);
-      if constexpr (!PBLK) {
-        p_pair_copy(pfill, pfill, pr + 2, c);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      p_pair_copy(pfill, pr + 2, c);
+      __builtin_amdgcn_sched_barrier(0);
       mma_one(1, 4 * c + 2);
       mma_one(1, 4 * c + 3);
       __builtin_amdgcn_sched_barrier(0);
@@ -261,13 +250,11 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   if (nkt > 0) {
     // weight pairs 0 and 1, activation pair 0; pair 0 has landed when the 8 copies of weight pair 1 are still in flight
 #pragma unroll
-    for (int j = 0; j < 8; ++j) p_pair_copy(ps0, PBLK ? ps1 : ps0, 0, j);
+    for (int j = 0; j < 8; ++j) p_pair_copy(ps0, 0, j);
 #pragma unroll
     for (int j = 0; j < 8; ++j) q_pair_copy(qs0, qs1, 0, j);
-    if constexpr (!PBLK) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) p_pair_copy(ps1, ps1, 1, j);
-    }
+    for (int j = 0; j < 8; ++j) p_pair_copy(ps1, 1, j);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(VM) : "memory");
 #pragma unroll
     for (int i = 0; i < 2 * NB; ++i) read_one(0, i, ps0, 0, qs0);
