@@ -212,7 +212,7 @@ def configs_leg(capi, torch, fsw_weights):
         rec = {"M": M, "d": d, "ff": ff, "dtype": "bf16" if dtype == torch.bfloat16 else "fp16", "calls": n,
                "ms_median": round(med, 5), "ms_p20": round(p20, 5), "ms_p80": round(p80, 5),
                "tflops": round(flops / med / 1e9, 2), "gbs": round(nbytes / med / 1e6, 2),
-               "kernels": "%s + %s" % (capi.variant_name(0, 0, M, 2 * ff, d), capi.variant_name(1, 0, M, d, ff))}
+               "kernels": "%s + %s" % (capi.variant_name(0, 0, M, 2 * ff, d), capi.variant_name(2, 0, M, d, ff))}
         if name == "C4":
             rec.update(bound="hbm", frac=round(nbytes / med / 1e6 / HBM_PEAK_GBS, 4))
         elif name == "C1":
@@ -347,7 +347,7 @@ def main():
     if hbm_bound:
         all_bytes = fsw_weights.hbm_bytes(M, d, ff)
         roofline = {"bound": "hbm", "kernel": "%s gate/up + %s down (whole forward, two launches)" % (
-                        capi.variant_name(0, 0, M, 2 * ff, d), capi.variant_name(1, 0, M, d, ff)),
+                        capi.variant_name(0, 0, M, 2 * ff, d), capi.variant_name(2, 0, M, d, ff)),
                     "achieved": round(all_bytes / (gu_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(all_bytes / (gu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                     "traffic": traffic, "traffic_source": traffic_src, "algorithmic_bytes": all_bytes,
@@ -400,7 +400,7 @@ def main():
         k4_ms, kc_ms = sum(k4) / len(k4), sum(kc) / len(kc)
         traffic4, traffic4_src = traffic_from_profile("C4")
         kern4 = "%s gate/up + %s down" % (capi.variant_name(0, 0, c4["M"], 2 * c4["ff"], c4["d"]),
-                                          capi.variant_name(1, 0, c4["M"], c4["d"], c4["ff"]))
+                                          capi.variant_name(2, 0, c4["M"], c4["d"], c4["ff"]))
         out["decode"] = {
             "workload": "C4: M=16 d=4096 ff=14336 bf16", "entry": "fsw_mlp (one call, two launches)",
             "warmup_steps": DECODE_WARMUP, "steps": 200,
