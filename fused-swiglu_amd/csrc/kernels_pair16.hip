@@ -287,6 +287,22 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   // two fragment sets, and the compiler would park them in scratch memory.
   const int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
   const int r16e = lane_e & 15, c4e = lane_e >> 4;
+  // Output stores are 16 bytes per lane: a lane's accumulator block holds 4 consecutive features (8 bytes), so two
+  // neighbouring 16-feature blocks (f, f + 1) are exchanged between the four 16-lane rows of the wave (lane = 16 c4 +
+  // r16) with two swap instructions per register -- upper/lower 32 lanes, then odd/even rows -- after which row c4
+  // holds features 8 (c4 & 1) .. + 7 of block f + (c4 >> 1): a store instruction then writes 64 contiguous bytes per
+  // activation row (a whole 1 KB run of the blocked layout) instead of 32.
+  auto widen = [](u32x2 lo, u32x2 hi) -> u32x4 {  // lo: block f, hi: block f + 1 (packed pairs of features)
+    u32x4 out;
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+      const auto s32 = __builtin_amdgcn_permlane32_swap(lo[d], hi[d], false, false);
+      const auto s16 = __builtin_amdgcn_permlane16_swap(s32[0], s32[1], false, false);
+      out[d] = s16[0];
+      out[2 + d] = s16[1];
+    }
+    return out;
+  };
   if constexpr (OBLK) {
     // H panel-blocked (see store_tile_blocked): every row of the panel and every feature up to the next multiple
     // of 32 is written; padding comes out of zero operand rows
@@ -296,15 +312,18 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     for (int g = 0; g < NB; ++g) {
       const int row = wq * 128 + g * 16 + r16e;
 #pragma unroll
-      for (int f = 0; f < NB / 2; ++f) {
+      for (int f = 0; f < NB / 2; f += 2) {
         const int blk = tp * 4 + wp * 2 + (f >> 1);
-        if (blk < nblocks) {
+        u32x2 pk[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
           float v[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = acc[f][g][e] * silu_f32(acc[f + NB / 2][g][e]);
-          u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
-          *(u32x2*)(O + (((long long)tq * nblocks + blk) * 256 + row) * 64 + (f & 1) * 32 + c4e * 8) = pk;
+          for (int e = 0; e < 4; ++e) v[e] = acc[f + h][g][e] * silu_f32(acc[f + h + NB / 2][g][e]);
+          pk[h] = u32x2{E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
         }
+        const u32x4 w = widen(pk[0], pk[1]);
+        if (blk < nblocks) *(u32x4*)(O + (((long long)tq * nblocks + blk) * 256 + row) * 64 + c4e * 16) = w;
       }
     }
   } else if constexpr (SPLIT) {
@@ -332,24 +351,37 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     constexpr int FO = GATED ? NB / 2 : NB;
     const int nout = GATED ? a.np / 2 : a.np;
     const bool vec_ok = ((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 7) == 0);
+    const bool vec16_ok = ((a.ldo & 7) == 0) && ((((uintptr_t)a.O) & 15) == 0);
+    const int nbase = GATED ? p0 / 2 + wp * 64 : p0 + wp * 128;
 #pragma unroll
     for (int g = 0; g < NB; ++g) {
       const int m = q0 + wq * 128 + g * 16 + r16e;
-      if (m >= a.nq) continue;
       unsigned short* orow = O + (long long)m * a.ldo;
 #pragma unroll
-      for (int f = 0; f < FO; ++f) {
-        const int n = (GATED ? p0 / 2 + wp * 64 : p0 + wp * 128) + f * 16 + c4e * 4;
-        float v[4];
+      for (int f = 0; f < FO; f += 2) {
+        float v[2][4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = GATED ? acc[f][g][e] * silu_f32(acc[f + FO][g][e]) : acc[f][g][e];
-        if (vec_ok && n + 3 < nout) {
-          u32x2 pk = {E::pack2(v[0], v[1]), E::pack2(v[2], v[3])};
-          *(u32x2*)(orow + n) = pk;
-        } else {
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (n + e < nout) orow[n + e] = E::cvt1(v[e]);
+            v[h][e] = GATED ? acc[f + h][g][e] * silu_f32(acc[f + h + FO][g][e]) : acc[f + h][g][e];
+        if (vec16_ok && nbase + (f + 2) * 16 <= nout) {  // wave-uniform: both blocks lie inside the matrix
+          const u32x4 w = widen(u32x2{E::pack2(v[0][0], v[0][1]), E::pack2(v[0][2], v[0][3])},
+                                u32x2{E::pack2(v[1][0], v[1][1]), E::pack2(v[1][2], v[1][3])});
+          if (m < a.nq) *(u32x4*)(orow + nbase + (f + (c4e >> 1)) * 16 + (c4e & 1) * 8) = w;
+        } else if (m < a.nq) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int n = nbase + (f + h) * 16 + c4e * 4;
+            if (vec_ok && n + 3 < nout) {
+              u32x2 pk = {E::pack2(v[h][0], v[h][1]), E::pack2(v[h][2], v[h][3])};
+              *(u32x2*)(orow + n) = pk;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (n + e < nout) orow[n + e] = E::cvt1(v[h][e]);
+            }
+          }
         }
       }
     }
