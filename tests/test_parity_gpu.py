@@ -113,6 +113,33 @@ def test_every_tiled_variant(capi, variant, dtype):
         capi.set_variant(1, -1)
 
 
+@pytest.mark.parametrize("pad", [0, 8, 4, 1])
+def test_large_tile_output_store_paths(capi, pad):
+    """The 256 x 256 kernel stores 16 bytes per lane when the output row stride and base allow it (pad 0, 8), 8 bytes
+    when only that alignment holds (pad 4) and single elements otherwise (pad 1); feature counts that end inside a
+    pair of 16-feature blocks take the narrow path for that pair. Outputs are column slices of wider NaN-filled
+    buffers, so a store past a row's end would show."""
+    M, d, ff = 300, 136, 200            # gated: 200 features = 6 whole block pairs + 8; plain: 136 = 4 pairs + 8
+    dtype = torch.bfloat16
+    inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=77 + pad, x_scale=0.5)
+    g = to_dev(inp)
+    try:
+        capi.set_variant(0, 5)
+        capi.set_variant(1, 5)
+        Hbig = torch.full((M, ff + pad), float("nan"), dtype=dtype, device=DEV)
+        H = capi.gateup(g["X"], g["W13"], out=Hbig[:, :ff])
+        assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "H pad %d" % pad)
+        assert pad == 0 or torch.isnan(Hbig[:, ff:]).all()
+        Ybig = torch.full((M, d + pad), float("nan"), dtype=dtype, device=DEV)
+        Hc = H.contiguous()
+        Y = capi.down(Hc, g["W2"], out=Ybig[:, :d])
+        assert_one_rounding(Y, oracle.ref_down(Hc.cpu(), inp["W2"], torch.float64), dtype, "Y pad %d" % pad)
+        assert pad == 0 or torch.isnan(Ybig[:, d:]).all()
+    finally:
+        capi.set_variant(0, -1)
+        capi.set_variant(1, -1)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [1, 7, 16, 17, 33, 48, 64])
 def test_skinny_weight_streaming_variant(capi, M, dtype):
