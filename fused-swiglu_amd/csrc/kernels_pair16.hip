@@ -26,7 +26,8 @@ typedef __attribute__((address_space(3))) void lds_void;
 // The main loop walks K in pairs with ONE workgroup barrier per pair (see pair_iteration); the slot/stage pattern
 // repeats every 6 pairs (lcm of 3 and 2), so the loop is unrolled sixfold with every LDS address a compile-time
 // constant. Measured against one barrier per K tile (copies three tiles ahead): gate/up 1.285 -> 1.270 ms at
-// 8192 x 4096 x 28672, bit-identical results (the K order is the same).
+// 8192 x 4096 x 28672, bit-identical results (the K order is the same); with the barrier in the middle of the pair
+// and reads and copies spread evenly over its quarters another 0.6 % (gate/up) and 1.6 % (down).
 // LDS layouts: pair slot = [256 rows][128 B], chunk c of row r at position c ^ ((r >> 1) & 7); activation stage =
 // [256 rows][64 B], chunk c at c ^ ((r >> 2) & 3): the 16 rows a fragment read touches at one logical chunk cover
 // the 64 banks once. The swizzle is applied on the global side of the copy (which lane fetches which chunk), since
@@ -145,13 +146,18 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
 
   // two register sets of the 16 fragments of a K tile: [0..7] weight blocks, [8..15] activation blocks
   u32x4 fr[2][2 * NB];
-  // ONE workgroup barrier per K PAIR (two K tiles, 128 MFMAs per wave). Pair iteration I works on tile a = 2I (fragments
-  // in register set 0) and tile b = 2I + 1 (set 1) in four quarters of 32 MFMAs:
-  //   Q1  a, weight blocks 0..3   + the 8 activation copies of pair I + 1 (its two stages were freed by barrier I - 1)
-  //   Q2  a, weight blocks 4..7   + the 16 fragment reads of b
-  //   Q3  b, weight blocks 0..3   + the 8 weight copies of pair I + 2 (into the slot of pair I - 1)
-  //   barrier: everything but the 8 copies of Q3 has landed (pair I + 1 complete); every wave has read a and b
-  //   Q4  b, weight blocks 4..7   + the 16 fragment reads of tile a of pair I + 1
+  // ONE workgroup barrier per K PAIR (two K tiles, 128 MFMAs per wave), in the MIDDLE of the pair. Pair iteration I
+  // multiplies tile a = 2I (fragments in register set 0) and tile b = 2I + 1 (set 1) in four quarters of 32 MFMAs;
+  // every quarter carries 8 fragment reads and 4 copies, so that LDS and the copy queue see an even load:
+  //   Q1  a, weight blocks 0..3   + the activation fragments of b      + weight copies 0..3 of pair I + 2
+  //   Q2  a, weight blocks 4..7   + the weight fragments of b (first half of the quarter) + weight copies 4..7
+  //   barrier: pair I + 1 has landed (all but the 8 weight copies just issued); every wave has read all of pair I
+  //   Q3  b, weight blocks 0..3   + the activation fragments of tile a of pair I + 1 + activation copies 0..3 of
+  //                                 pair I + 2 (into the two stages of pair I, free since the barrier)
+  //   Q4  b, weight blocks 4..7   + the weight fragments of tile a of pair I + 1     + activation copies 4..7
+  // The weight copies of pair I + 2 go into the slot pair I - 1 left at the previous barrier. Measured at
+  // 8192 x 4096 x 14336 against the barrier at the end of Q3 (16 reads in Q2 and in Q4, 8 copies in Q1 and in Q3):
+  // gate/up -0.6 %, down -1.6 %; weight copies issued a pair earlier still (in Q4): down +3.7 %.
   constexpr int VM = 2 * LPH;
   constexpr int WAIT_IMM = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
   auto read_one = [&](int set, int idx, const unsigned char* pslot, int half, const unsigned char* qstage) {
@@ -199,63 +205,83 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     constexpr int I = decltype(i_c)::value;  // pair index modulo 6: LDS addresses are compile-time constants
     unsigned char* const pb = ps[I % 3] + (PBLK ? PSTAGE : 0);  // tile b of this pair
     unsigned char* const pna = ps[(I + 1) % 3];                 // tile a of the next pair
-    unsigned char* const pfill = ps[(I + 2) % 3];
-    unsigned char* const qa = qs[(2 * I) & 3];
+    unsigned char* const pfill = ps[(I + 2) % 3];               // slot of pair I - 1: refilled with pair I + 2
+    unsigned char* const qfa = qs[(2 * I) & 3];  // stages of this pair: refilled with pair I + 2 after the barrier
     unsigned char* const qb = qs[(2 * I + 1) & 3];
     unsigned char* const qna = qs[(2 * I + 2) & 3];
-    unsigned char* const qnb = qs[(2 * I + 3) & 3];
-    (void)qa;
-    // Q1
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
       mma_one(0, 4 * c + 0);
+      read_one(1, 1 + c, pb, 1, qb);
       mma_one(0, 4 * c + 1);
-      q_pair_copy(qna, qnb, pr + 1, c);
       __builtin_amdgcn_sched_barrier(0);
       mma_one(0, 4 * c + 2);
+      if (c & 1) {
+        p_pair_copy(pfill, pr + 2, c >> 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       mma_one(0, 4 * c + 3);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // Q2
-#pragma unroll
-    for (int r = 0; r < 2 * NB; ++r) {
-      mma_one(0, 4 * NB + 2 * r);
-      read_one(1, r, pb, 1, qb);
-      mma_one(0, 4 * NB + 2 * r + 1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // Q3
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
-      mma_one(1, 4 * c + 0);
-      mma_one(1, 4 * c + 1);
-      p_pair_copy(pfill, pr + 2, c);
+      mma_one(0, 4 * NB + 2 * c);
+      read_one(1, c == 0 ? 0 : NB + c, pb, 1, qb);
+      mma_one(0, 4 * NB + 2 * c + 1);
       __builtin_amdgcn_sched_barrier(0);
-      mma_one(1, 4 * c + 2);
-      mma_one(1, 4 * c + 3);
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      mma_one(0, 4 * NB + 16 + 4 * c);
+      mma_one(0, 4 * NB + 16 + 4 * c + 1);
+      p_pair_copy(pfill, pr + 2, 4 + c);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_one(0, 4 * NB + 16 + 4 * c + 2);
+      mma_one(0, 4 * NB + 16 + 4 * c + 3);
       __builtin_amdgcn_sched_barrier(0);
     }
     asm volatile("s_waitcnt %0\n\ts_barrier" ::"n"(WAIT_IMM) : "memory");
-    // Q4
 #pragma unroll
-    for (int r = 0; r < 2 * NB; ++r) {
-      mma_one(1, 4 * NB + 2 * r);
-      read_one(0, r, pna, 0, qna);
-      mma_one(1, 4 * NB + 2 * r + 1);
+    for (int c = 0; c < 8; ++c) {
+      mma_one(1, 4 * c + 0);
+      read_one(0, 1 + c, pna, 0, qna);
+      mma_one(1, 4 * c + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_one(1, 4 * c + 2);
+      if (c & 1) {
+        q_pair_copy(qfa, qb, pr + 2, c >> 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mma_one(1, 4 * c + 3);
       __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      mma_one(1, 4 * NB + 4 * c);
+      read_one(0, c == 0 ? 0 : NB + c, pna, 0, qna);
+      mma_one(1, 4 * NB + 4 * c + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_one(1, 4 * NB + 4 * c + 2);
+      if (c & 1) {
+        q_pair_copy(qfa, qb, pr + 2, 4 + (c >> 1));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mma_one(1, 4 * NB + 4 * c + 3);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
   if (nkt > 0) {
-    // weight pairs 0 and 1, activation pair 0; pair 0 has landed when the 8 copies of weight pair 1 are still in flight
+    // pairs 0 and 1 of both operands; pair 0 has landed when the 16 copies of pair 1 are still in flight
 #pragma unroll
     for (int j = 0; j < 8; ++j) p_pair_copy(ps0, 0, j);
 #pragma unroll
     for (int j = 0; j < 8; ++j) q_pair_copy(qs0, qs1, 0, j);
 #pragma unroll
     for (int j = 0; j < 8; ++j) p_pair_copy(ps1, 1, j);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(VM) : "memory");
+#pragma unroll
+    for (int j = 0; j < 8; ++j) q_pair_copy(qs2, qs3, 1, j);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * VM) : "memory");
 #pragma unroll
     for (int i = 0; i < 2 * NB; ++i) read_one(0, i, ps0, 0, qs0);
   }
