@@ -113,6 +113,32 @@ def test_every_tiled_variant(capi, variant, dtype):
         capi.set_variant(1, -1)
 
 
+def _random_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    return [(int(rng.integers(65, 700)), int(rng.integers(1, 70)) * 8, int(rng.integers(1, 70)) * 8) for _ in range(n)]
+
+
+@pytest.mark.parametrize("shape", _random_shapes(10, 20240607))
+def test_large_tile_kernel_on_random_ragged_shapes(capi, shape):
+    """The 256 x 256 kernel forced onto shapes it is never picked for: every combination of ragged rows, ragged
+    features and K that is no multiple of 64 or even of 32 goes through its zero-filling copies, its K-pair loop
+    tails (1 .. 9 pairs) and its narrow store paths. Both projections, against the fp64 oracle."""
+    M, d, ff = shape
+    dtype = torch.bfloat16 if (M + d + ff) % 2 else torch.float16
+    inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=M * 7 + d + ff, x_scale=0.5)
+    g = to_dev(inp)
+    try:
+        capi.set_variant(0, 5)
+        capi.set_variant(1, 5)
+        H = capi.gateup(g["X"], g["W13"])
+        assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "H %s" % (shape,))
+        Y = capi.down(H, g["W2"])
+        assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype, "Y %s" % (shape,))
+    finally:
+        capi.set_variant(0, -1)
+        capi.set_variant(1, -1)
+
+
 @pytest.mark.parametrize("pad", [0, 8, 4, 1])
 def test_large_tile_output_store_paths(capi, pad):
     """The 256 x 256 kernel stores 16 bytes per lane when the output row stride and base allow it (pad 0, 8), 8 bytes
