@@ -37,6 +37,9 @@ sys.path.insert(0, os.path.join(ROOT, "fused-swiglu_amd"))
 MFMA_PEAK_TFLOPS = 2516.6  # MI355X dense bf16/fp16: 256 CU x 2.4 GHz x 4096 flop/clk/CU
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 DECODE_WARMUP = 500        # untimed forwards before the HBM-bound (M = 16) measurements, ~30 ms
+SETTLE_MS = 60.0           # untimed forwards before the timed steps of the compute-bound legs, whatever --warmup says:
+                           # after an idle period the board's clock needs ~25 ms of load to settle (the reference's
+                           # timer, bench_swiglu.py:102-106, warms up for about as long)
 FLUSH_BYTES = 512 << 20    # written before every timed call of the per-configuration leg (Infinity Cache: 256 MB)
 # counter profiles (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measurable in-process) that hold the line
 # `traffic_bytes_per_launch = N` for the dominant kernel of a workload
@@ -74,18 +77,20 @@ def traffic_from_profile(workload):
     return (int(m.group(1)), rel) if m else (None, None)
 
 
-def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False, prepacked=False, weight_sets=None):
+def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False, prepacked=False, weight_sets=None, settle_ms=0.0):
     """Times exactly `steps` forwards between two device synchronisations.
     fused_entry=False: a step is the launch sequence fsw_mlp enqueues for this shape, issued through the
     per-step entry points so that HIP events can be recorded around each launch inside the timed region: in the
-    large-tile regime fsw_block_rows(X) -> fsw_gateup_blocked -> fsw_down_blocked (H stays blocked in the
-    workspace), otherwise fsw_gateup -> fsw_down. prepacked=True passes weights blocked once, outside the timed
-    region, by fsw_prepack_w13 / fsw_prepack_w2.
+    large-tile regime fsw_gateup_hblocked -> fsw_down_blocked (X row-major, H blocked in the workspace), otherwise
+    fsw_gateup -> fsw_down. prepacked=True passes weights blocked once, outside the timed region, by
+    fsw_prepack_w13 / fsw_prepack_w2.
     fused_entry=True: a step is one fsw_mlp call and ONE event pair brackets the whole timed region (an event
     record costs the stream ~4 us, which is 6 % of a 64 us decode step but 0.2 % of a prefill step); the per-step
     kernel time is then the bracketed time / steps, inter-launch gaps included. weight_sets: a list of (W13, W2)
     pairs used round-robin, step by step.
-    Returns (wall seconds, [ms of gate/up], [ms of down], Y, [ms of the X re-block or 0])."""
+    settle_ms: untimed steps are issued until at least this much device time has gone by (and at least `warmup`).
+    Returns (wall seconds, [ms of gate/up], [ms of down], Y, [0.0], info) with info =
+    {"settle_steps", "settle_ms", "step_ms": per-step device time from the step's first to its last event}."""
     import fsw_capi
     L = capi.lib()
     M, d, ff = cfg["M"], cfg["d"], cfg["ff"]
@@ -95,8 +100,7 @@ def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False, prepacked=F
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=g["X"].device)
     h_bytes = (M * ff * 2 + 255) // 256 * 256
     hb_bytes = L.fsw_blocked_bytes(M, ff)
-    blocked = (not fused_entry) and capi.variant_name(0, code, M, 2 * ff, d) == "pair16_256x256" and \
-        ws_bytes == hb_bytes + L.fsw_blocked_bytes(M, d)
+    blocked = (not fused_entry) and capi.variant_name(0, code, M, 2 * ff, d) == "pair16_256x256" and ws_bytes == hb_bytes
     stream = torch.cuda.current_stream().cuda_stream
     xp, wp, w2p, yp, wsp = (t.data_ptr() for t in (g["X"], g["W13"], g["W2"], Y, ws))
     sets = [(a.data_ptr(), b.data_ptr()) for a, b in weight_sets] if weight_sets else [(wp, w2p)]
@@ -113,13 +117,12 @@ def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False, prepacked=F
             rc = L.fsw_mlp(code, M, d, ff, xp, d, a, d, b, ff, yp, d, wsp, ws_bytes, stream)
             rc2 = rc3 = 0
         elif blocked:
-            ev[3].record()
-            rc3 = L.fsw_block_rows(code, M, d, xp, d, wsp + hb_bytes, stream)
             ev[0].record()
-            rc = L.fsw_gateup_blocked(code, M, 2 * ff, d, wsp + hb_bytes, wp, ldw, wflag, wsp, 0, stream)
+            rc = L.fsw_gateup_hblocked(code, M, 2 * ff, d, xp, d, wp, ldw, wflag, wsp, stream)
             ev[1].record()
             rc2 = L.fsw_down_blocked(code, M, d, ff, wsp, w2p, ldw2, wflag, yp, d, stream)
             ev[2].record()
+            rc3 = 0
         else:
             ev[0].record()
             rc = L.fsw_gateup(code, M, 2 * ff, d, xp, d, wp, d, wsp, ff, stream)
@@ -132,8 +135,17 @@ def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False, prepacked=F
 
     events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps + min(warmup, 16))]
     region = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-    for i in range(warmup):
-        step(events[steps + i % min(warmup, 16)], i)
+    spare = events[steps:] or [[torch.cuda.Event(enable_timing=True) for _ in range(4)]]
+    settle = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    settle[0].record()
+    done, settled = 0, 0.0
+    while done < warmup or settled < settle_ms:
+        for _ in range(8 if done >= warmup else min(8, warmup - done)):
+            step(spare[done % len(spare)], done)
+            done += 1
+        settle[1].record()
+        settle[1].synchronize()
+        settled = settle[0].elapsed_time(settle[1])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     region[0].record()
@@ -142,12 +154,13 @@ def run_steps(capi, torch, g, cfg, steps, warmup, fused_entry=False, prepacked=F
     region[1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    info = {"settle_steps": done, "settle_ms": round(settled, 2), "blocked": blocked}
     if fused_entry:
-        return wall, [region[0].elapsed_time(region[1]) / steps], [0.0], Y, [0.0]
+        return wall, [region[0].elapsed_time(region[1]) / steps], [0.0], Y, [0.0], info
     first = [e[0].elapsed_time(e[1]) for e in events[:steps]]
     second = [e[1].elapsed_time(e[2]) for e in events[:steps]]
-    pre = [e[3].elapsed_time(e[0]) for e in events[:steps]] if blocked else [0.0]
-    return wall, first, second, Y, pre
+    info["step_ms"] = [e[0].elapsed_time(e[2]) for e in events[:steps]]
+    return wall, first, second, Y, [0.0], info
 
 
 def quantiles(xs):
@@ -226,19 +239,47 @@ def configs_leg(capi, torch, fsw_weights):
     return out
 
 
-def comparator_leg(torch, g, cfg, fsw_weights):
-    """hipBLASLt through torch.mm on the two GEMM shapes of the workload (no gating, C written at full width)."""
+def comparator_leg(torch, g, cfg, fsw_weights, steps, warmup, settle_ms):
+    """hipBLASLt through torch.mm on the two GEMM shapes of the workload (no gating, C written at full width), timed
+    the way `value` is: the same settling period and warm-up steps, then exactly `steps` back-to-back pairs of GEMMs
+    between two device synchronisations, events around each GEMM inside the timed region."""
     M, d, ff = cfg["M"], cfg["d"], cfg["ff"]
     X, W13, W2 = g["X"], g["W13"], g["W2"]
     C = torch.empty((M, 2 * ff), dtype=X.dtype, device=X.device)
     H = torch.randn((M, ff), device=X.device).to(X.dtype)
     Y = torch.empty((M, d), dtype=X.dtype, device=X.device)
     w13t, w2t = W13.t(), W2.t()
-    gu = timed_calls(torch, lambda: torch.mm(X, w13t, out=C), None, min_calls=20, budget_ms=100.0)
-    dn = timed_calls(torch, lambda: torch.mm(H, w2t, out=Y), None, min_calls=20, budget_ms=100.0)
-    both = gu[0] + dn[0]
-    return {"what": "torch.mm (hipBLASLt) on the gate/up [M,d]x[d,2ff] and down [M,ff]x[ff,d] shapes, back-to-back "
-                    "calls, no gating kernel, no flush",
+
+    def step(ev):
+        ev[0].record()
+        torch.mm(X, w13t, out=C)
+        ev[1].record()
+        torch.mm(H, w2t, out=Y)
+        ev[2].record()
+
+    mk = lambda: [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    spare, settle = mk(), [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    settle[0].record()
+    done, settled = 0, 0.0
+    while done < warmup or settled < settle_ms:
+        for _ in range(8 if done >= warmup else min(8, warmup - done)):
+            step(spare)
+            done += 1
+        settle[1].record()
+        settle[1].synchronize()
+        settled = settle[0].elapsed_time(settle[1])
+    events = [mk() for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for ev in events:
+        step(ev)
+    torch.cuda.synchronize()
+    both = (time.perf_counter() - t0) / steps * 1e3
+    gu = quantiles([e[0].elapsed_time(e[1]) for e in events])
+    dn = quantiles([e[1].elapsed_time(e[2]) for e in events])
+    return {"what": "torch.mm (hipBLASLt) on the gate/up [M,d]x[d,2ff] and down [M,ff]x[ff,d] shapes, no gating kernel; "
+                    "timed like `value`: %.0f ms (%d steps) of settling, then %d back-to-back steps between two "
+                    "synchronisations" % (settled, done, steps),
             "gateup_ms_median": round(gu[0], 5), "gateup_tflops": round(4 * M * d * ff / gu[0] / 1e9, 2),
             "down_ms_median": round(dn[0], 5), "down_tflops": round(2 * M * d * ff / dn[0] / 1e9, 2),
             "two_gemms_ms": round(both, 5), "two_gemms_tflops": round(fsw_weights.flops(M, d, ff) / both / 1e9, 2)}
@@ -280,9 +321,21 @@ def ceilings_leg(capi, torch):
                           "(beyond the 256 MB Infinity Cache) per launch"}
 
 
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(torch, inp, cfg, passes, y_gpu):
     """The fp32 PyTorch formulation on the host cores: one warm-up block, then `passes` whole forwards of the
-    workload. The last result is the reference for a parity check of every row of the GPU's Y."""
+    workload. The last result is the reference for a parity check of every row of the GPU's Y. `cores` is the
+    number of threads torch actually runs (OMP_NUM_THREADS where the host sets it: a one-GPU share of a larger
+    machine), `host_cpus` what the machine shows."""
     from oracle import oracle
     import fsw_weights
     M, d, ff = cfg["M"], cfg["d"], cfg["ff"]
@@ -299,7 +352,7 @@ def cpu_baseline(torch, inp, cfg, passes, y_gpu):
     parity["rows"] = M
     parity["pass"] = bool(oracle.passes(parity))
     base = {"value": round(fsw_weights.flops(M, d, ff) / med / 1e12, 4), "unit": "TFLOP/s", "cores": threads,
-            "kind": "port",
+            "host_cpus": os.cpu_count(), "cpu_model": cpu_model(), "kind": "port",
             "sample": "%d whole forwards of %s (all %d rows) by the fp32 torch formulation, median %.2f s of %s" % (
                 len(times), cfg["name"], M, med, ["%.2f" % t for t in times])}
     return base, parity
@@ -335,9 +388,11 @@ def main():
     # is at least DECODE_WARMUP steps of ~60 us.
     if hbm_bound:
         args.warmup = max(args.warmup, DECODE_WARMUP)
-    wall, gu, dn, Y, pre = run_steps(capi, torch, g, cfg, args.steps, args.warmup, fused_entry=hbm_bound)
+    settle_ms = 0.0 if hbm_bound else SETTLE_MS
+    wall, gu, dn, Y, pre, info = run_steps(capi, torch, g, cfg, args.steps, args.warmup, fused_entry=hbm_bound,
+                                           settle_ms=settle_ms)
     pre_ms = sum(pre) / len(pre)
-    blocked = pre_ms > 0
+    blocked = info["blocked"]
     ms_per_step = wall / args.steps * 1e3
     tflops = fsw_weights.flops(M, d, ff) / (ms_per_step * 1e-3) / 1e12
     gu_ms, dn_ms = sum(gu) / len(gu), max(sum(dn) / len(dn), 1e-9)
@@ -353,7 +408,7 @@ def main():
                     "traffic": traffic, "traffic_source": traffic_src, "algorithmic_bytes": all_bytes,
                     "avg_kernel_ms": round(gu_ms, 5)}
     else:
-        kname = capi.variant_name(0, 0, M, 2 * ff, d) + (" (v_mfma_f32_16x16x32), X and H panel-blocked" if blocked else "")
+        kname = capi.variant_name(0, 0, M, 2 * ff, d) + (" (v_mfma_f32_16x16x32), X row-major, H panel-blocked" if blocked else "")
         roofline = {"bound": "mfma", "kernel": kname + " (gate/up)",
                     "achieved": round(gu_tflops, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(gu_tflops / MFMA_PEAK_TFLOPS, 4),
@@ -364,14 +419,16 @@ def main():
     out = {
         "metric": "fused SwiGLU fwd TFLOP/s + %% bf16 MFMA peak (M=%d,d=%d,ff=%d)" % (M, d, ff),
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 5),
+        "ms_per_step_median": round(quantiles(info["step_ms"])[0], 5) if "step_ms" in info else round(ms_per_step, 5),
+        "settle_ms": info["settle_ms"], "settle_steps": info["settle_steps"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype_name, "data": "synthetic",
         "config": {"workload": "%s: SwiGLU MLP forward M=%d d=%d ff=%d %s seed %d" % (
             cfg["name"], M, d, ff, dtype_name, cfg["seed"]), "M": M, "d": d, "ff": ff},
         "frac_of_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS, 4),
         "kernels": {"gateup_ms": round(gu_ms, 5), "gateup_ms_median": round(quantiles(gu)[0], 5),
                     "gateup_tflops": round(gu_tflops, 2), "down_ms": round(dn_ms, 5),
-                    "down_tflops": round(dn_tflops, 2), "block_x_ms": round(pre_ms, 5),
+                    "down_tflops": round(dn_tflops, 2),
                     "hbm_gbs": round(fsw_weights.hbm_bytes(M, d, ff) / (ms_per_step * 1e-3) / 1e9, 2)},
         "roofline": roofline,
     }
@@ -384,7 +441,7 @@ def main():
         del src, dst
 
     if not hbm_bound and not args.no_comparator:
-        out["comparator"] = comparator_leg(torch, g, cfg, fsw_weights)
+        out["comparator"] = comparator_leg(torch, g, cfg, fsw_weights, args.steps, args.warmup, settle_ms)
         out["comparator"]["value_over_two_gemms"] = round(tflops / out["comparator"]["two_gemms_tflops"], 4)
 
     # decode leg: M = 16, weight streaming, judged in GB/s: steady state on one set of weights, and cold
@@ -394,8 +451,8 @@ def main():
         c4 = {"name": "C4", "M": tup[1], "d": tup[2], "ff": tup[3], "seed": tup[5]}
         g4 = {"X": X4, "W13": sets4[0][0], "W2": sets4[0][1]}
         by4 = fsw_weights.hbm_bytes(c4["M"], c4["d"], c4["ff"])
-        wall4, k4, _, _, _ = run_steps(capi, torch, g4, c4, 200, DECODE_WARMUP, fused_entry=True)
-        wallc, kc, _, _, _ = run_steps(capi, torch, g4, c4, 201, DECODE_WARMUP, fused_entry=True, weight_sets=sets4)
+        wall4, k4, _, _, _, _ = run_steps(capi, torch, g4, c4, 200, DECODE_WARMUP, fused_entry=True)
+        wallc, kc, _, _, _, _ = run_steps(capi, torch, g4, c4, 201, DECODE_WARMUP, fused_entry=True, weight_sets=sets4)
         ms4, msc = wall4 / 200 * 1e3, wallc / 201 * 1e3
         k4_ms, kc_ms = sum(k4) / len(k4), sum(kc) / len(kc)
         traffic4, traffic4_src = traffic_from_profile("C4")
@@ -427,12 +484,12 @@ def main():
     # the same forward with the weights blocked once, offline (fsw_prepack_w13 / fsw_prepack_w2): reported beside
     # `value`, which stays on the reference's weight layout
     if blocked and not args.no_prepacked:
-        wallp, gup, dnp, Yp, prep = run_steps(capi, torch, g, cfg, args.steps, args.warmup, prepacked=True)
+        wallp, gup, dnp, Yp, prep, _ = run_steps(capi, torch, g, cfg, args.steps, args.warmup, prepacked=True,
+                                                 settle_ms=settle_ms)
         msp = wallp / args.steps * 1e3
         out["prepacked_weights"] = {
             "ms_per_step": round(msp, 5), "value": round(fsw_weights.flops(M, d, ff) / (msp * 1e-3) / 1e12, 2),
             "unit": "TFLOP/s", "gateup_ms": round(sum(gup) / len(gup), 5), "down_ms": round(sum(dnp) / len(dnp), 5),
-            "block_x_ms": round(sum(prep) / len(prep), 5),
             "max_abs_vs_row_major_weights": round((Yp.float() - Y.float()).abs().max().item(), 6)}
 
     if not args.no_configs:

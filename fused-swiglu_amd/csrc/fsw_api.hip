@@ -186,8 +186,6 @@ int fsw_set_variant(int family, int variant) {
   return FSW_OK;
 }
 
-static bool down_reblock_wanted(int64_t M, int64_t D, int64_t FF);
-
 static fsw::StreamPlan mlp_stream_plan(int64_t M, int64_t D, int64_t FF);
 
 const char* fsw_variant_name(int family, int dtype, int64_t M, int64_t N_or_D, int64_t K_or_FF) {
@@ -311,19 +309,9 @@ static size_t stream_scratch_bytes(const fsw::StreamPlan& p) {
   return (p.partial_bytes + (size_t)p.ticket_words * 4 + 255) & ~(size_t)255;
 }
 
-// Row-major H in the large-tile regime: with scratch for a blocked copy of H the down projection runs the pair-ring
-// kernel on whole-line requests (8192 x 14336 x 4096: 0.10 ms of re-blocking + 0.62 ms against 0.80 ms for the
-// two-stage kernel on row-major H). Same rule for ragged panel counts as fsw_gateup_workspace_bytes.
-static bool down_reblock_wanted(int64_t M, int64_t D, int64_t FF) {
-  if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[1] >= 0 || pick_tiled(1, M, D) != V_256x256) return false;  // 129 tiles or more
-  if (M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM || fsw::tiled_split_plan((int)D, (int)M, (int)FF).splits > 1) return false;
-  return M >= 1024 || M % 256 == 0;
-}
-
 size_t fsw_down_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
   (void)dtype;
   if (M <= 0 || M > MAX_DIM || D <= 0 || D > MAX_DIM || FF <= 0 || FF > MAX_DIM || streams_weights(1, M, D, FF)) return 0;
-  if (down_reblock_wanted(M, D, FF)) return (size_t)fsw::blocked_bytes(M, FF);
   if (g_forced_variant[1] >= 0) return 0;  // a forced kernel runs unsplit
   const fsw::SplitPlan plan = fsw::tiled_split_plan((int)D, (int)M, (int)FF);
   return plan.splits > 1 ? (size_t)plan.splits * (size_t)M * (size_t)D * sizeof(float) : 0;
@@ -334,16 +322,7 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
   const int rc = fsw_validate_down(dtype, M, D, FF, H, ldh, W2, ldw2, Y, ldy);
   if (rc != FSW_OK) return rc;
   if (M == 0 || D == 0) return FSW_OK;
-  size_t need = fsw_down_workspace_bytes(dtype, M, D, FF);
-  if (down_reblock_wanted(M, D, FF)) {
-    // the blocked copy is an optimisation: without scratch the row-major kernel below runs instead
-    if (workspace && workspace_bytes >= need && aligned16(workspace)) {
-      const int brc = fsw_block_rows(dtype, M, FF, H, ldh, workspace, stream);
-      if (brc != FSW_OK) return brc;
-      return fsw_down_blocked(dtype, M, D, FF, workspace, W2, ldw2, 0, Y, ldy, stream);
-    }
-    need = 0;
-  }
+  const size_t need = fsw_down_workspace_bytes(dtype, M, D, FF);
   if (need > 0 && (!workspace || workspace_bytes < need)) return FSW_E_WORKSPACE;
   const int drc = check_device();
   if (drc != FSW_OK) return drc;
@@ -384,8 +363,9 @@ int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF, const void* H, int64_t
   return finish(fsw::launch_tiled(v, dtype, false, a, (hipStream_t)stream));
 }
 
-// Large-tile regime of fsw_mlp: both projections run 256 x 256 tiles, so X is re-blocked once into the workspace
-// and H never exists row-major (the gate/up epilogue writes it blocked, the down projection reads it blocked).
+// Large-tile regime of fsw_mlp: both projections run 256 x 256 tiles, and H never exists row-major: the gate/up
+// epilogue writes it panel-blocked (whole 1 KB runs) and the down projection reads it blocked. Against row-major H
+// the whole forward measures 0.8 % (8192 x 4096 x 14336) to 1.3 % (4096 x 4096 x 11008) faster; X is read row-major.
 static bool blocked_regime(int64_t M, int64_t D, int64_t FF) {
   if (M <= 64 || D <= 0 || FF <= 0 || g_forced_variant[0] >= 0 || g_forced_variant[1] >= 0) return false;
   if (M > MAX_DIM || D > MAX_DIM || FF > MAX_DIM / 2) return false;
@@ -455,6 +435,30 @@ int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* X
   return finish(fsw::launch_pair16(dtype, true, a, (hipStream_t)stream));
 }
 
+int fsw_gateup_hblocked(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13,
+                        int64_t ldw, int w_blocked, void* Hb, void* stream) {
+  // blocked weights have no leading dimension: validated as if their rows were K long
+  const int rc = fsw_validate_gateup(dtype, M, N, K, X, ldx, W13, w_blocked ? K : ldw, Hb, N / 2);
+  if (rc != FSW_OK) return rc;
+  if (M == 0 || N == 0) return FSW_OK;
+  if (K == 0) return FSW_E_SHAPE;  // a blocked matrix with no columns has no representation
+  if (!aligned16(Hb)) return FSW_E_ALIGN;
+  const int drc = check_device();
+  if (drc != FSW_OK) return drc;
+  fsw::GemmArgs a;
+  a.P = W13;
+  a.Q = X;
+  a.O = Hb;
+  a.ldp = ldw;
+  a.ldq = ldx;
+  a.ldo = 0;
+  a.np = (int)N;
+  a.nq = (int)M;
+  a.k = (int)K;
+  a.layout = w_blocked ? 6 : 2;
+  return finish(fsw::launch_pair16(dtype, true, a, (hipStream_t)stream));
+}
+
 int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* Hb, const void* W2, int64_t ldw2,
                      int w_blocked, void* Y, int64_t ldy, void* stream) {
   if (dtype != FSW_BF16 && dtype != FSW_FP16) return FSW_E_DTYPE;
@@ -482,31 +486,22 @@ int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* Hb
   return finish(fsw::launch_pair16(dtype, false, a, (hipStream_t)stream));
 }
 
-// fsw_gateup with caller scratch: in the large-tile regime X is re-blocked into the scratch first (the gated
-// kernel then reads whole cache lines: 1.52 -> 1.40 + 0.03 ms at 8192 x 4096 x 28672); H stays row-major.
+// fsw_gateup never needs scratch: the large-tile kernel reads row-major X in whole cache lines (K pairs), which
+// measures level with a blocked copy of X (8192 x 4096 x 28672: 1.2515 vs 1.2530 ms) and saves the copy. The two
+// entry points stay for callers written against them.
 size_t fsw_gateup_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K) {
   (void)dtype;
-  if (M <= 64 || N <= 0 || K <= 0 || M > MAX_DIM || N > MAX_DIM || K > MAX_DIM) return 0;  // large tiles only
-  if (g_forced_variant[0] >= 0 || pick_tiled(0, M, N) != V_256x256) return 0;
-  // Few activation panels with a ragged last one: the re-block launch and the zero rows of the padded panel (read
-  // from memory, where the row-major kernel's out-of-range rows cost no traffic) outweigh the whole-line requests.
-  // Measured at 4096 x 28672, blocked vs row-major ring: M = 384: 145 vs 129 us, 576: 215 vs 190, 640: 216 vs 199,
-  // 896: 222 vs 211, 960: 223 vs 219; M = 512: 141 vs 147, 1024: 226 vs 241, 1152: level, 1536: 310 vs 329.
-  if (M < 1024 && M % 256 != 0) return 0;
-  return (size_t)fsw::blocked_bytes(M, K);
+  (void)M;
+  (void)N;
+  (void)K;
+  return 0;
 }
 
 int fsw_gateup_ws(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13, int64_t ldw,
                   void* H, int64_t ldh, void* workspace, size_t workspace_bytes, void* stream) {
-  const size_t want = fsw_gateup_workspace_bytes(dtype, M, N, K);
-  if (want == 0 || !workspace || workspace_bytes < want || !aligned16(workspace)) {
-    return fsw_gateup(dtype, M, N, K, X, ldx, W13, ldw, H, ldh, stream);
-  }
-  int rc = fsw_validate_gateup(dtype, M, N, K, X, ldx, W13, ldw, H, ldh);
-  if (rc != FSW_OK) return rc;
-  rc = fsw_block_rows(dtype, M, K, X, ldx, workspace, stream);
-  if (rc != FSW_OK) return rc;
-  return fsw_gateup_blocked(dtype, M, N, K, workspace, W13, ldw, 0, H, ldh, stream);
+  (void)workspace;
+  (void)workspace_bytes;
+  return fsw_gateup(dtype, M, N, K, X, ldx, W13, ldw, H, ldh, stream);
 }
 
 static size_t h_bytes(int64_t M, int64_t FF) {
@@ -516,12 +511,11 @@ static size_t h_bytes(int64_t M, int64_t FF) {
 
 size_t fsw_mlp_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF) {
   if (M <= 0 || D <= 0 || FF <= 0) return 0;
-  if (blocked_regime(M, D, FF)) return (size_t)fsw::blocked_bytes(M, FF) + (size_t)fsw::blocked_bytes(M, D);
+  if (blocked_regime(M, D, FF)) return (size_t)fsw::blocked_bytes(M, FF);  // H, panel-blocked
   const fsw::StreamPlan sp = mlp_stream_plan(M, D, FF);
   if (sp.splits > 1) return h_bytes(M, FF) + stream_scratch_bytes(sp);  // [H row-major][partials][ticket counters]
-  // otherwise [H row-major][split-K scratch of the down projection][X blocked, when gate/up alone runs large tiles]
-  return h_bytes(M, FF) + ((fsw_down_workspace_bytes(dtype, M, D, FF) + 255) & ~(size_t)255) +
-         fsw_gateup_workspace_bytes(dtype, M, 2 * FF, D);
+  // otherwise [H row-major][split-K scratch of the down projection]
+  return h_bytes(M, FF) + ((fsw_down_workspace_bytes(dtype, M, D, FF) + 255) & ~(size_t)255);
 }
 
 // single_launch_ok: whether the opt-in single-launch decode forward may be used (it creates events on first use,
@@ -570,14 +564,10 @@ static int mlp_impl(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, 
       if (lrc != FSW_OK || launched) return lrc;
     }
   }
-  if (blocked_regime(M, D, FF)) {  // workspace = [H blocked][X blocked]
-    unsigned char* Hb = (unsigned char*)workspace;
-    unsigned char* Xb = Hb + fsw::blocked_bytes(M, FF);
-    rc = fsw_block_rows(dtype, M, D, X, ldx, Xb, stream);
+  if (blocked_regime(M, D, FF)) {  // workspace = H, panel-blocked
+    rc = fsw_gateup_hblocked(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, 0, workspace, stream);
     if (rc != FSW_OK) return rc;
-    rc = fsw_gateup_blocked(dtype, M, 2 * FF, D, Xb, W13, ldw13, 0, Hb, 0, stream);
-    if (rc != FSW_OK) return rc;
-    return fsw_down_blocked(dtype, M, D, FF, Hb, W2, ldw2, 0, Y, ldy, stream);
+    return fsw_down_blocked(dtype, M, D, FF, workspace, W2, ldw2, 0, Y, ldy, stream);
   }
   unsigned char* ws2 = (unsigned char*)workspace + h_bytes(M, FF);
   const fsw::StreamPlan sp = mlp_stream_plan(M, D, FF);
@@ -598,8 +588,7 @@ static int mlp_impl(int dtype, int64_t M, int64_t D, int64_t FF, const void* X, 
     return finish(fsw::launch_stream_split(dtype, a, sp, ws2, (hipStream_t)stream));
   }
   const size_t down_ws = (fsw_down_workspace_bytes(dtype, M, D, FF) + 255) & ~(size_t)255;
-  rc = fsw_gateup_ws(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF, ws2 + down_ws,
-                     fsw_gateup_workspace_bytes(dtype, M, 2 * FF, D), stream);
+  rc = fsw_gateup(dtype, M, 2 * FF, D, X, ldx, W13, ldw13, Hbuf, FF, stream);
   if (rc != FSW_OK) return rc;
   return fsw_down(dtype, M, D, FF, Hbuf, FF, W2, ldw2, Y, ldy, ws2, down_ws, stream);
 }

@@ -37,8 +37,10 @@ typedef __attribute__((address_space(3))) void lds_void;
 // PBLK: the weight operand is panel-blocked as well (prepacked; for the gated kernel in de-interleaved row order). It
 // then arrives like the activations, one 16 KB block per K tile; a pair slot holds the two blocks of a K pair, one
 // after the other, as 64-byte rows, and the ring of three slots runs on the same schedule as for row-major weights.
-// QROW: the activation operand is row-major (callers without scratch for a blocked copy; few ragged activation
-// panels, where re-blocking does not pay): 64-byte requests per row and K tile, rows past nq read as zero.
+// QROW: the activation operand is row-major as well (no blocked copy of it exists anywhere). It is then fetched
+// exactly like row-major weights, in K pairs of one whole 128-byte line per row, into TWO pair slots that take the
+// place of the four stages (same 64 KB, same schedule: the slot of pair I is free from the barrier of pair I on and
+// is refilled with pair I + 2); rows past nq read as zero.
 // SPLIT (row-major operands, plain product): blockIdx.y selects one of a.splits contiguous runs of 64-element K
 // pairs; the workgroup multiplies that run only and stores its fp32 accumulators to a.partial[blockIdx.y][nq][np].
 template <class E, bool GATED, bool KTAIL, bool OBLK, bool PBLK = false, bool QROW = false, bool SPLIT = false>
@@ -61,16 +63,23 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   constexpr int LPH = 4;  // weight copy instructions per wave per HALF pair (8 rows x 128 B each)
   constexpr int LQ = 4;   // activation copy instructions per wave per K tile (16 rows x 64 B each)
   static_assert(!OBLK || GATED, "only H is ever written blocked");
-  static_assert(!PBLK || !KTAIL, "blocked operands are zero padded in K");
+  static_assert(!PBLK || !KTAIL || QROW, "blocked operands are zero padded in K");
   constexpr int PSTAGE = BP * 64;
 
   __shared__ __align__(1024) unsigned char ps0[PSLOT];
   __shared__ __align__(1024) unsigned char ps1[PSLOT];
   __shared__ __align__(1024) unsigned char ps2[PSLOT];
-  __shared__ __align__(1024) unsigned char qs0[QSTAGE];
-  __shared__ __align__(1024) unsigned char qs1[QSTAGE];
-  __shared__ __align__(1024) unsigned char qs2[QSTAGE];
-  __shared__ __align__(1024) unsigned char qs3[QSTAGE];
+  // activations: four 16 KB stages, or (QROW) two 32 KB pair slots qs0, qs1; one array per stage or slot
+  __shared__ __align__(1024) unsigned char qs0[QROW ? PSLOT : QSTAGE];
+  __shared__ __align__(1024) unsigned char qs1[QROW ? PSLOT : QSTAGE];
+  unsigned char* qs2 = nullptr;
+  unsigned char* qs3 = nullptr;
+  if constexpr (!QROW) {  // 160 KB are all there is: the two stages exist only where they are used
+    __shared__ __align__(1024) unsigned char qs2_mem[QSTAGE];
+    __shared__ __align__(1024) unsigned char qs3_mem[QSTAGE];
+    qs2 = qs2_mem;
+    qs3 = qs3_mem;
+  }
   unsigned char* const ps[3] = {ps0, ps1, ps2};
   unsigned char* const qs[4] = {qs0, qs1, qs2, qs3};
 
@@ -110,15 +119,15 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   const int pcq = t & 3;
   const int rbq = t >> 2;
   const int lcq = pcq ^ ((rbq >> 2) & 3);
-  static_assert(!(QROW && (PBLK || OBLK)), "row-major activations: row-major weights and output only");
   const unsigned char* qbase = QROW ? (const unsigned char*)a.Q + (long long)q0 * a.ldq * 2
                                     : (const unsigned char*)a.Q + (long long)tq * nkt * QSTAGE;
   const __amdgpu_buffer_rsrc_t qrs =
       make_rsrc(qbase, QROW ? ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2 : (long long)nkt * QSTAGE);
-  // Activation copy j covers rows rbq + 64 j. Blocked panels are zero padded and need no bounds check: the j and K
-  // parts go into the scalar offset. Row-major activations (QROW) are treated like the weights.
+  // Activation copy j covers rows rbq + 64 j of one K tile. Blocked panels are zero padded and need no bounds check:
+  // the j and K parts go into the scalar offset. Row-major activations (QROW) are treated like row-major weights:
+  // copy j covers rows rbp + 32 j of a K pair.
   const unsigned ldq2 = (unsigned)a.ldq * 2u;
-  const unsigned qoff0 = QROW ? (unsigned)rbq * ldq2 + (unsigned)lcq * 16u : (unsigned)rbq * 64u + (unsigned)lcq * 16u;
+  const unsigned qoff0 = QROW ? (unsigned)rbp * ldq2 + (unsigned)lcp * 16u : (unsigned)rbq * 64u + (unsigned)lcq * 16u;
   auto p_copy = [&](lds_void* dst, int j, int pair, bool in) {  // row-major weights: copy j (0 .. 7) of a K pair
     const unsigned voff = poff0 + (p_row_off(j) + (unsigned)pair * 128u);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(prs, dst, 16, (int)(in ? voff : OOB_OFFSET), 0, 0, 0);
@@ -128,7 +137,8 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
   const unsigned rd_p = PBLK ? (unsigned)((GATED ? wp * 64 : wp * 128) + r16) * 64u +
                                    (unsigned)((c4 ^ ((r16 >> 2) & 3)) * 16)
                              : (unsigned)((GATED ? wp * 64 : wp * 128) + r16) * 128u;
-  const unsigned rd_q = (unsigned)(wq * 128 + r16) * 64u + (unsigned)((c4 ^ ((r16 >> 2) & 3)) * 16);
+  const unsigned rd_q = QROW ? (unsigned)(wq * 128 + r16) * 128u
+                             : (unsigned)(wq * 128 + r16) * 64u + (unsigned)((c4 ^ ((r16 >> 2) & 3)) * 16);
   unsigned xp[2];  // [half of the pair]
 #pragma unroll
   for (int h = 0; h < 2; ++h) xp[h] = (unsigned)((((h << 2) | c4) ^ ((r16 >> 1) & 7)) * 16);
@@ -164,7 +174,7 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     if (idx == 0) {
       fr[set][0] = *(const u32x4*)(pslot + rd_p + p_block_off(0) + (PBLK ? 0u : xp[half]));
     } else if (idx <= NB) {
-      fr[set][NB + idx - 1] = *(const u32x4*)(qstage + rd_q + (idx - 1) * 16 * 64);
+      fr[set][NB + idx - 1] = *(const u32x4*)(qstage + rd_q + (idx - 1) * 16 * (QROW ? 128 : 64) + (QROW ? xp[half] : 0u));
     } else {
       fr[set][idx - NB] = *(const u32x4*)(pslot + rd_p + p_block_off(idx - NB) + (PBLK ? 0u : xp[half]));
     }
@@ -173,17 +183,19 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     E::mfma16_acc(acc[i / NB][i % NB], fr[set][i / NB], fr[set][NB + i % NB]);
   };
   // activation copy j (0 .. 7) of pair `pair`: tile 2 pair + j / 4; tiles past the end arrive as zeros
+  // (QROW: st_a is the pair slot, st_b unused; copy j covers rows 32 j .. 32 j + 31 of the pair, 128 bytes each)
   auto q_pair_copy = [&](unsigned char* st_a, unsigned char* st_b, int pair, int j) {
-    const int qt = 2 * pair + j / LQ;
-    unsigned char* st = j < LQ ? st_a : st_b;
-    lds_void* dst = (lds_void*)(st + (j % LQ) * 64 * 64 + wave * 1024);
-    const bool qin = qt < nkt && (!(QROW && KTAIL) || (qt * 32 + lcq * 8) < a.k);
     if constexpr (QROW) {
-      const unsigned voff = qoff0 + ((unsigned)((j % LQ) * 64) * ldq2 + (unsigned)qt * 64u);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, dst, 16, (int)(qin ? voff : OOB_OFFSET), 0, 0, 0);
+      const bool qin = pair < npair && (!KTAIL || (pair * 64 + lcp * 8) < a.k);
+      const unsigned voff = qoff0 + ((unsigned)(32 * j) * ldq2 + (unsigned)pair * 128u);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, (lds_void*)(st_a + j * 32 * 128 + wave * 1024), 16,
+                                               (int)(qin ? voff : OOB_OFFSET), 0, 0, 0);
     } else {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, dst, 16, (int)(qin ? qoff0 : OOB_OFFSET), (j % LQ) * 64 * 64 + qt * QSTAGE, 0,
-                                               0);
+      const int qt = 2 * pair + j / LQ;
+      unsigned char* st = j < LQ ? st_a : st_b;
+      lds_void* dst = (lds_void*)(st + (j % LQ) * 64 * 64 + wave * 1024);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(qrs, dst, 16, (int)(qt < nkt ? qoff0 : OOB_OFFSET),
+                                               (j % LQ) * 64 * 64 + qt * QSTAGE, 0, 0);
     }
   };
   // weight copy j (0 .. 7) of pair `pair` into a pair slot: row-major: 32 rows of 128 bytes; prepacked: a quarter of
@@ -206,9 +218,10 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
     unsigned char* const pb = ps[I % 3] + (PBLK ? PSTAGE : 0);  // tile b of this pair
     unsigned char* const pna = ps[(I + 1) % 3];                 // tile a of the next pair
     unsigned char* const pfill = ps[(I + 2) % 3];               // slot of pair I - 1: refilled with pair I + 2
-    unsigned char* const qfa = qs[(2 * I) & 3];  // stages of this pair: refilled with pair I + 2 after the barrier
-    unsigned char* const qb = qs[(2 * I + 1) & 3];
-    unsigned char* const qna = qs[(2 * I + 2) & 3];
+    // stages (QROW: the slot) of this pair: refilled with pair I + 2 after the barrier
+    unsigned char* const qfa = QROW ? qs[I & 1] : qs[(2 * I) & 3];
+    unsigned char* const qb = QROW ? qs[I & 1] : qs[(2 * I + 1) & 3];
+    unsigned char* const qna = QROW ? qs[(I + 1) & 1] : qs[(2 * I + 2) & 3];
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
       mma_one(0, 4 * c + 0);
@@ -280,7 +293,7 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
 #pragma unroll
     for (int j = 0; j < 8; ++j) p_pair_copy(ps1, 1, j);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) q_pair_copy(qs2, qs3, 1, j);
+    for (int j = 0; j < 8; ++j) q_pair_copy(QROW ? qs1 : qs2, qs3, 1, j);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * VM) : "memory");
 #pragma unroll
     for (int i = 0; i < 2 * NB; ++i) read_one(0, i, ps0, 0, qs0);
@@ -433,18 +446,18 @@ hipError_t launch_pair16_blocked_x(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// both operands row-major
-template <class E, bool GATED>
+// both operands row-major (OBLK: H written blocked)
+template <class E, bool GATED, bool OBLK = false>
 hipError_t launch_pair16_rowmajor(const GemmArgs& a, hipStream_t stream) {
   const int tiles_p = (a.np + 255) / 256;
   const int tiles_q = (a.nq + 255) / 256;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
   const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
   if (a.k % 64 == 0) {
-    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, false, false, true>), grid, block, 0, stream, a, tiles_p,
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK, false, true>), grid, block, 0, stream, a, tiles_p,
                        tiles_q, raster_group(GATED, tiles_q));
   } else {
-    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, false, false, true>), grid, block, 0, stream, a, tiles_p,
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, OBLK, false, true>), grid, block, 0, stream, a, tiles_p,
                        tiles_q, raster_group(GATED, tiles_q));
   }
   return hipGetLastError();
@@ -467,14 +480,20 @@ hipError_t launch_pair16_split(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// both operands blocked (prepacked weights): the 16x16x32 kernel with a stage ring for the weights
-template <class E, bool GATED, bool OBLK>
+// weights blocked (prepacked): a stage ring for the weights; activations blocked, or (QROW) row-major in K pairs
+template <class E, bool GATED, bool OBLK, bool QROW = false>
 hipError_t launch_pair16_blocked_xw(const GemmArgs& a, hipStream_t stream) {
   const int tiles_p = (a.np + 255) / 256;
   const int tiles_q = (a.nq + 255) / 256;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
-  hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK, true>), dim3((unsigned)(tiles_p * tiles_q)), dim3(256), 0,
-                     stream, a, tiles_p, tiles_q, raster_group(GATED, tiles_q));
+  const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
+  if (!QROW || a.k % 64 == 0) {  // blocked activations are zero padded in K; row-major ones need the K-tail checks
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK, true, QROW>), grid, block, 0, stream, a, tiles_p,
+                       tiles_q, raster_group(GATED, tiles_q));
+  } else if constexpr (QROW) {
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, OBLK, true, QROW>), grid, block, 0, stream, a, tiles_p,
+                       tiles_q, raster_group(GATED, tiles_q));
+  }
   return hipGetLastError();
 }
 
@@ -486,6 +505,8 @@ hipError_t launch_pair16_typed(bool gated, const GemmArgs& a, hipStream_t stream
   if (gated && a.layout == 5) return launch_pair16_blocked_xw<E, true, false>(a, stream);
   if (gated && a.layout == 7) return launch_pair16_blocked_xw<E, true, true>(a, stream);
   if (!gated && a.layout == 5) return launch_pair16_blocked_xw<E, false, false>(a, stream);
+  if (gated && a.layout == 2) return launch_pair16_rowmajor<E, true, true>(a, stream);
+  if (gated && a.layout == 6) return launch_pair16_blocked_xw<E, true, true, true>(a, stream);
   if (a.layout == 0) return gated ? launch_pair16_rowmajor<E, true>(a, stream) : launch_pair16_rowmajor<E, false>(a, stream);
   return hipErrorInvalidValue;
 }

@@ -53,12 +53,9 @@ void swiglu_fwd_typed(at::ScalarType want, int64_t m, int64_t n, int64_t k, Tens
     TORCH_CHECK(C.numel() >= (m - 1) * (ldC / 2) + n / 2, "tensor C is smaller than m x n/2 with row stride ldC/2");
   }
   const at::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(A));
-  // large problems: scratch for a blocked copy of A lets the kernel fetch whole cache lines (same result)
-  const size_t ws_bytes = fsw_gateup_workspace_bytes(dtype_code(want), m, n, k);
-  Tensor ws;
-  if (ws_bytes > 0) ws = at::empty({(int64_t)ws_bytes}, A.options().dtype(at::kByte));
-  const int rc = fsw_gateup_ws(dtype_code(want), m, n, k, A.data_ptr(), ldA, B.data_ptr(), ldB, C.data_ptr(), ldC / 2,
-                               ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, current_stream());
+  // like the reference's launcher this allocates nothing: the kernels read A and B where they lie
+  const int rc = fsw_gateup(dtype_code(want), m, n, k, A.data_ptr(), ldA, B.data_ptr(), ldB, C.data_ptr(), ldC / 2,
+                            current_stream());
   check_rc(rc, "swiglu_fwd");
 }
 

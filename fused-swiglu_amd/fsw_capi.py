@@ -31,6 +31,7 @@ PROTOTYPES = {
     "fsw_prepack_w13": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
     "fsw_prepack_w2": (_i, [_i, _i64, _i64, _vp, _i64, _vp, _vp]),
     "fsw_gateup_blocked": (_i, [_i, _i64, _i64, _i64, _vp, _vp, _i64, _i, _vp, _i64, _vp]),
+    "fsw_gateup_hblocked": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _i, _vp, _vp]),
     "fsw_down_blocked": (_i, [_i, _i64, _i64, _i64, _vp, _vp, _i64, _i, _vp, _i64, _vp]),
     "fsw_gateup_workspace_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "fsw_gateup_ws": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
@@ -275,6 +276,23 @@ def gateup_blocked(Xb, W13, row_major_out=False):
     with torch.cuda.device(like.device):
         check(lib().fsw_gateup_blocked(code, Xb.rows, N, Xb.k, Xb.data_ptr(), W13.data_ptr(), 0 if wb else _ld(W13),
                                        1 if wb else 0, H.data_ptr(), ldh, _stream(like)))
+    return H
+
+
+def gateup_hblocked(X, W13):
+    """Gate/up of a row-major X written as a Blocked H (what fsw_mlp runs in the large-tile regime). W13: row-major
+    tensor or a Blocked from block_rows(W13, "w13")."""
+    import torch
+    _check_operands(X)
+    wb = isinstance(W13, Blocked)
+    if not wb:
+        _check_operands(X, W13)
+    N = W13.rows if wb else W13.shape[0]
+    M, K = X.shape
+    H = _blocked_empty(M, N // 2, X)
+    with torch.cuda.device(X.device):
+        check(lib().fsw_gateup_hblocked(dtype_code(X), M, N, K, X.data_ptr(), _ld(X), W13.data_ptr(),
+                                        0 if wb else _ld(W13), 1 if wb else 0, H.data_ptr(), _stream(X)))
     return H
 
 

@@ -82,10 +82,8 @@ FSW_API int fsw_validate_down(int dtype, int64_t M, int64_t D, int64_t FF,
                       const void* H, int64_t ldh, const void* W2, int64_t ldw2,
                       const void* Y, int64_t ldy);
 
-/* Bytes of device scratch fsw_down uses for this shape: fp32 split-K partials in the small-M regime (required:
- * FSW_E_WORKSPACE without them), a panel-blocked copy of H in the large-tile regime (optional: without it the kernel
- * for row-major H runs, about 10 % slower), 0 otherwise. No counterpart in the reference, which has no down
- * projection. */
+/* Bytes of device scratch fsw_down needs for this shape: fp32 split-K partials where few output tiles meet a deep K
+ * (FSW_E_WORKSPACE without them), 0 otherwise. No counterpart in the reference, which has no down projection. */
 FSW_API size_t fsw_down_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF);
 
 /*
@@ -98,7 +96,8 @@ FSW_API int fsw_down(int dtype, int64_t M, int64_t D, int64_t FF,
              void* Y, int64_t ldy,
              void* workspace, size_t workspace_bytes, void* stream);
 
-/* Bytes of device scratch fsw_mlp needs: the H[M, FF] intermediate plus fsw_down's scratch. */
+/* Bytes of device scratch fsw_mlp needs: the H[M, FF] intermediate (panel-blocked in the large-tile regime) plus the
+ * scratch of its down projection. */
 FSW_API size_t fsw_mlp_workspace_bytes(int dtype, int64_t M, int64_t D, int64_t FF);
 
 /*
@@ -134,9 +133,9 @@ FSW_API const char* fsw_strerror(int code);
  * large-tile kernels fetch whole cache lines). A blocked copy of a row-major [rows, k] matrix is ceil(rows / 256)
  * panels of ceil(k / 32) blocks; block (panel, kt) is [256 rows][32 elements] contiguous (16 KB) and holds rows
  * 256 panel .. 256 panel + 255, columns 32 kt .. 32 kt + 31, zero padded. fsw_mlp uses it internally for M > 64 when
- * both projections run 256 x 256 tiles (X re-blocked into the workspace, H written and read blocked); the entry
- * points below expose the steps, and let a caller block the weights ONCE (fsw_prepack_*) and pass them with
- * w_blocked = 1. Constraints as for fsw_gateup / fsw_down (K, FF and row-major leading dimensions multiples of 8,
+ * both projections run 256 x 256 tiles: H is written and read blocked (fsw_gateup_hblocked, fsw_down_blocked); X is
+ * read row-major. The entry points below expose the steps, and let a caller block the weights ONCE (fsw_prepack_*)
+ * and pass them with w_blocked = 1. Constraints as for fsw_gateup / fsw_down (K, FF and row-major leading dimensions multiples of 8,
  * 16-byte aligned bases); the blocked kernels are the 256 x 256 tiled kernels, whatever M is.
  */
 FSW_API size_t fsw_blocked_bytes(int64_t rows, int64_t k);
@@ -152,13 +151,17 @@ FSW_API int fsw_prepack_w2(int dtype, int64_t D, int64_t FF, const void* W2, int
  * written blocked when ldh == 0 (for fsw_down_blocked), else row-major with row stride ldh. */
 FSW_API int fsw_gateup_blocked(int dtype, int64_t M, int64_t N, int64_t K, const void* X_blocked, const void* W13,
                                int64_t ldw, int w_blocked, void* H, int64_t ldh, void* stream);
+/* fsw_gateup on row-major X (row stride ldx) whose H is written blocked, for fsw_down_blocked: the two halves of
+ * fsw_mlp in the large-tile regime. W13 row-major (w_blocked = 0, ldw) or from fsw_prepack_w13 (1). K > 0;
+ * constraints as for fsw_gateup; H 16-byte aligned. */
+FSW_API int fsw_gateup_hblocked(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13,
+                                int64_t ldw, int w_blocked, void* H_blocked, void* stream);
 /* Y[M, D] (row-major, ldy) = H_blocked[M, FF] @ W2^T; W2 row-major (0, ldw2) or from fsw_prepack_w2 (1). */
 FSW_API int fsw_down_blocked(int dtype, int64_t M, int64_t D, int64_t FF, const void* H_blocked, const void* W2,
                              int64_t ldw2, int w_blocked, void* Y, int64_t ldy, void* stream);
 
-/* fsw_gateup with optional scratch (same arguments, same result): with at least fsw_gateup_workspace_bytes() of
- * 16-byte aligned scratch the large-tile regime re-blocks X into it first; with none (or for other shapes, where
- * the query returns 0) it is fsw_gateup. */
+/* fsw_gateup with a scratch argument, kept for callers written against it: the query returns 0 for every shape and
+ * the call is fsw_gateup (the large-tile kernel reads row-major X in whole cache lines; no blocked copy is made). */
 FSW_API size_t fsw_gateup_workspace_bytes(int dtype, int64_t M, int64_t N, int64_t K);
 FSW_API int fsw_gateup_ws(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13,
                           int64_t ldw, void* H, int64_t ldh, void* workspace, size_t workspace_bytes, void* stream);

@@ -148,9 +148,12 @@ def test_variant_choice_by_regime(capi):
     assert name(1, 2304, 4096, 14336) == "pair16_256x256"    # 144 large tiles in one round: no split
     # 288 large tiles of a very deep K: three splits (four rounds of K / 3 instead of two of K), H stays row-major
     assert name(1, 2049, 8192, 28672) == "splitk_pair16_256x256" and ws(0, 2049, 8192, 28672) == 3 * 2049 * 8192 * 4
-    # large-tile regime: scratch for a blocked copy of H (optional: without it fsw_down runs on row-major H)
-    assert ws(0, 8192, 4096, 14336) == L.fsw_blocked_bytes(8192, 14336) == 8192 * 14336 * 2
-    assert ws(0, 3000, 4096, 14336) == L.fsw_blocked_bytes(3000, 14336) and ws(0, 16, 4096, 14336) == 0
+    # large-tile regime: fsw_down reads row-major H in whole cache lines and needs no scratch; fsw_gateup never does;
+    # fsw_mlp keeps H panel-blocked between its two kernels and nothing else
+    assert ws(0, 8192, 4096, 14336) == 0 and ws(0, 3000, 4096, 14336) == 0 and ws(0, 16, 4096, 14336) == 0
+    assert L.fsw_gateup_workspace_bytes(0, 8192, 28672, 4096) == 0
+    assert L.fsw_mlp_workspace_bytes(0, 8192, 4096, 14336) == L.fsw_blocked_bytes(8192, 14336) == 8192 * 14336 * 2
+    assert L.fsw_mlp_workspace_bytes(0, 3000, 4096, 14336) == L.fsw_blocked_bytes(3000, 14336)
     assert capi.lib().fsw_mlp_workspace_bytes(0, 256, 4096, 14336) == 256 * 14336 * 2 + ws(0, 256, 4096, 14336)
 
 

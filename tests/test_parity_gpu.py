@@ -661,6 +661,10 @@ def test_blocked_kernels_against_oracle(capi, dtype, prepacked):
         # row-major H straight from the blocked X: the same bits as the blocked H
         Hrm = capi.gateup_blocked(Xb, W13, row_major_out=True)
         assert torch.equal(Hrm, H)
+        # blocked H straight from the row-major X (the form fsw_mlp runs): the same bits again
+        Hb2 = capi.gateup_hblocked(g["X"], W13)
+        assert torch.equal(capi.unblock(Hb2), H)
+        assert torch.equal(capi.down_blocked(Hb2, W2), Y)
         # against the row-major kernels: the same products, summed in the same K order by the same kernel
         H2 = capi.gateup(g["X"], g["W13"])
         assert (H.float() - H2.float()).abs().max().item() <= 2 * ulp_rel(dtype) * 2 * H2.float().abs().max().item() + 1e-3
@@ -684,19 +688,39 @@ def test_blocked_kernels_take_strided_row_major_operands(capi):
 
 
 def test_mlp_large_tile_regime_uses_blocked_path(capi):
-    """For M > 64 with both projections on 256 x 256 tiles fsw_mlp re-blocks X into the workspace and keeps H blocked;
-    the result agrees with the separate row-major entry points and with the oracle, and the workspace query covers
-    both blocked buffers."""
+    """For M > 64 with both projections on 256 x 256 tiles fsw_mlp reads X where it lies and keeps H panel-blocked
+    between its two kernels; the result equals that of the separate row-major entry points bit for bit (the K order
+    is the same) and agrees with the oracle, and the workspace query covers the blocked H and nothing else."""
     M, d, ff = 4096, 4096, 2048
     L = capi.lib()
-    assert L.fsw_mlp_workspace_bytes(0, M, d, ff) == L.fsw_blocked_bytes(M, ff) + L.fsw_blocked_bytes(M, d)
+    assert L.fsw_mlp_workspace_bytes(0, M, d, ff) == L.fsw_blocked_bytes(M, ff)
+    assert L.fsw_gateup_workspace_bytes(0, M, 2 * ff, d) == 0 and L.fsw_down_workspace_bytes(0, M, d, ff) == 0
     inp = fsw_weights.make_inputs(M, d, ff, torch.bfloat16, seed=99, x_scale=0.5)
     g = to_dev(inp)
     Y = capi.mlp(g["X"], g["W13"], g["W2"])
     Y2 = capi.down(capi.gateup(g["X"], g["W13"]), g["W2"])
     rows = torch.arange(0, M, 37)
     oracle.assert_parity(Y[rows.to(DEV)], oracle.ref_mlp(inp["X"][rows], inp["W13"], inp["W2"], torch.float64), "mlp blocked regime")
-    assert (Y.float() - Y2.float()).abs().max().item() <= 2e-2
+    assert torch.equal(Y, Y2)
+    # the two halves through their own entry points: row-major X -> blocked H -> Y
+    Hb = torch.empty(L.fsw_blocked_bytes(M, ff), dtype=torch.uint8, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    capi.check(L.fsw_gateup_hblocked(0, M, 2 * ff, d, g["X"].data_ptr(), d, g["W13"].data_ptr(), d, 0, Hb.data_ptr(), stream))
+    Y3 = torch.empty_like(Y)
+    capi.check(L.fsw_down_blocked(0, M, d, ff, Hb.data_ptr(), g["W2"].data_ptr(), ff, 0, Y3.data_ptr(), d, stream))
+    assert torch.equal(Y3, Y)
+    # a ragged problem with strided X: rows past M and the K tail come out of the bounds check, not of memory
+    M2, d2, ff2 = 700, 1064, 520
+    inp = fsw_weights.make_inputs(M2, d2, ff2, torch.float16, seed=98, x_scale=0.5)
+    g = to_dev(inp)
+    Xs = torch.full((M2, d2 + 24), float("nan"), dtype=torch.float16, device=DEV)
+    Xs[:, :d2] = g["X"]
+    Hb = torch.full((L.fsw_blocked_bytes(M2, ff2),), 0xFF, dtype=torch.uint8, device=DEV)
+    capi.check(L.fsw_gateup_hblocked(1, M2, 2 * ff2, d2, Xs.data_ptr(), d2 + 24, g["W13"].data_ptr(), d2, 0, Hb.data_ptr(), stream))
+    Y4 = torch.empty((M2, d2), dtype=torch.float16, device=DEV)
+    capi.check(L.fsw_down_blocked(1, M2, d2, ff2, Hb.data_ptr(), g["W2"].data_ptr(), ff2, 0, Y4.data_ptr(), d2, stream))
+    oracle.assert_parity(Y4, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64), "hblocked ragged fp16")
+    assert torch.equal(Y4, capi.down(capi.gateup(g["X"], g["W13"]), g["W2"]))
 
 
 @pytest.mark.parametrize("shape", [(16, 512, 1024), (96, 512, 1024), (600, 1024, 520)])
