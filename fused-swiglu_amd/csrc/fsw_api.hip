@@ -287,6 +287,32 @@ int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_
   return gateup_impl(dtype, M, N, K, X, ldx, W13, ldw, H, ldh, stream, nullptr, 0);
 }
 
+// The reference's other build (C_TYPE float, constants.cuh:9-14; "C can work with either bf16 or fp32",
+// swiglu.cu:470-471): H is float and receives the gated fp32 value without a rounding. Two kernels serve it: the
+// weight-streaming kernel up to 64 rows, the 256 x 256 kernel on row-major operands above.
+int fsw_gateup_f32out(int dtype, int64_t M, int64_t N, int64_t K, const void* X, int64_t ldx, const void* W13,
+                      int64_t ldw, float* H, int64_t ldh, void* stream) {
+  const int rc = fsw_validate_gateup(dtype, M, N, K, X, ldx, W13, ldw, H, ldh);
+  if (rc != FSW_OK) return rc;
+  if (M == 0 || N == 0) return FSW_OK;
+  if ((((uintptr_t)H) & 3)) return FSW_E_ALIGN;
+  const int drc = check_device();
+  if (drc != FSW_OK) return drc;
+  fsw::GemmArgs a;
+  a.P = W13;
+  a.Q = X;
+  a.O = H;
+  a.ldp = ldw;
+  a.ldq = ldx;
+  a.ldo = ldh;
+  a.np = (int)N;
+  a.nq = (int)M;
+  a.k = (int)K;
+  a.out_f32 = 1;
+  if (M <= 64) return finish(fsw::launch_skinny(dtype, true, a, nullptr, (hipStream_t)stream));
+  return finish(fsw::launch_pair16(dtype, true, a, (hipStream_t)stream));
+}
+
 // Inside fsw_mlp the down projection of up to 32 activation rows runs the split-K streaming kernel when (i) the
 // gate/up product before it runs a kernel that zeroes the ticket counters (skinny_kernel or the 128 x 64 tiled
 // kernel), (ii) the down projection is in the weight-streaming regime and (iii) the shape is large enough for the

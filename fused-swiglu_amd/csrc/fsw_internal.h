@@ -28,6 +28,9 @@ struct GemmArgs {
   // skinny_kernel honour it): the ticket counters of the split-K streaming down projection that follows in fsw_mlp
   unsigned* zero_words = nullptr;
   int n_zero_words = 0;
+  // gated kernels on row-major operands (skinny_kernel, the 256 x 256 kernel with layout 0): O is float [nq, np/2]
+  // and receives the gated fp32 value unrounded (the reference's build with C_TYPE float, constants.cuh:9)
+  int out_f32 = 0;
 };
 inline long long blocked_bytes(long long rows, long long k) {
   return ((rows + 255) / 256) * ((k + 31) / 32) * (256 * 64);

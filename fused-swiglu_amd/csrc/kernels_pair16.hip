@@ -43,10 +43,13 @@ typedef __attribute__((address_space(3))) void lds_void;
 // is refilled with pair I + 2); rows past nq read as zero.
 // SPLIT (row-major operands, plain product): blockIdx.y selects one of a.splits contiguous runs of 64-element K
 // pairs; the workgroup multiplies that run only and stores its fp32 accumulators to a.partial[blockIdx.y][nq][np].
-template <class E, bool GATED, bool KTAIL, bool OBLK, bool PBLK = false, bool QROW = false, bool SPLIT = false>
+// OF32 (gated, row-major operands and output): H is float and receives the gated value unrounded.
+template <class E, bool GATED, bool KTAIL, bool OBLK, bool PBLK = false, bool QROW = false, bool SPLIT = false,
+          bool OF32 = false>
 __global__ void __launch_bounds__(256)
 tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, const int group) {
   static_assert(!SPLIT || (QROW && !GATED && !OBLK && !PBLK), "split-K: row-major operands, plain product");
+  static_assert(!OF32 || (GATED && QROW && !OBLK && !PBLK), "fp32 output: the gated kernel on row-major operands");
   GemmArgs a = a_in;
   if constexpr (SPLIT) {  // the run of this workgroup as a product of its own: shifted operands, shorter K
     const int per = ((a_in.k + 63) / 64 + a_in.splits - 1) / a_in.splits * 64;
@@ -385,6 +388,31 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
         }
       }
     }
+  } else if constexpr (OF32) {
+    float* O = (float*)a.O;
+    const int nout = a.np / 2;
+    const bool vec_ok = ((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 15) == 0);
+    const int nbase = p0 / 2 + wp * 64;
+#pragma unroll
+    for (int g = 0; g < NB; ++g) {
+      const int m = q0 + wq * 128 + g * 16 + r16e;
+      if (m >= a.nq) continue;
+      float* orow = O + (long long)m * a.ldo;
+#pragma unroll
+      for (int f = 0; f < NB / 2; ++f) {
+        f32x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[f][g][e] * silu_f32(acc[f + NB / 2][g][e]);
+        const int n = nbase + f * 16 + c4e * 4;
+        if (vec_ok && n + 3 < nout) {
+          *(f32x4*)(orow + n) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < nout) orow[n + e] = v[e];
+        }
+      }
+    }
   } else {
     unsigned short* O = (unsigned short*)a.O;
     constexpr int FO = GATED ? NB / 2 : NB;
@@ -446,19 +474,19 @@ hipError_t launch_pair16_blocked_x(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// both operands row-major (OBLK: H written blocked)
-template <class E, bool GATED, bool OBLK = false>
+// both operands row-major (OBLK: H written blocked; OF32: H float)
+template <class E, bool GATED, bool OBLK = false, bool OF32 = false>
 hipError_t launch_pair16_rowmajor(const GemmArgs& a, hipStream_t stream) {
   const int tiles_p = (a.np + 255) / 256;
   const int tiles_q = (a.nq + 255) / 256;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
   const dim3 grid((unsigned)(tiles_p * tiles_q)), block(256);
   if (a.k % 64 == 0) {
-    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK, false, true>), grid, block, 0, stream, a, tiles_p,
-                       tiles_q, raster_group(GATED, tiles_q));
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, false, OBLK, false, true, false, OF32>), grid, block, 0, stream, a,
+                       tiles_p, tiles_q, raster_group(GATED, tiles_q));
   } else {
-    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, OBLK, false, true>), grid, block, 0, stream, a, tiles_p,
-                       tiles_q, raster_group(GATED, tiles_q));
+    hipLaunchKernelGGL((tiled_pair16_kernel<E, GATED, true, OBLK, false, true, false, OF32>), grid, block, 0, stream, a,
+                       tiles_p, tiles_q, raster_group(GATED, tiles_q));
   }
   return hipGetLastError();
 }
@@ -507,6 +535,8 @@ hipError_t launch_pair16_typed(bool gated, const GemmArgs& a, hipStream_t stream
   if (!gated && a.layout == 5) return launch_pair16_blocked_xw<E, false, false>(a, stream);
   if (gated && a.layout == 2) return launch_pair16_rowmajor<E, true, true>(a, stream);
   if (gated && a.layout == 6) return launch_pair16_blocked_xw<E, true, true, true>(a, stream);
+  if (gated && a.layout == 0 && a.out_f32) return launch_pair16_rowmajor<E, true, false, true>(a, stream);
+  if (a.out_f32) return hipErrorInvalidValue;
   if (a.layout == 0) return gated ? launch_pair16_rowmajor<E, true>(a, stream) : launch_pair16_rowmajor<E, false>(a, stream);
   return hipErrorInvalidValue;
 }

@@ -192,6 +192,17 @@ skinny_kernel(const GemmArgs a) {
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = GATED ? sum[0][e] * silu_f32(sum[T - 1][e]) : sum[0][e];
+      if (GATED && a.out_f32) {  // H as float, unrounded
+        float* orow32 = (float*)a.O + (long long)m * a.ldo;
+        if (((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 15) == 0) && n + 3 < nout) {
+          *(f32x4*)(orow32 + n) = f32x4{v[0], v[1], v[2], v[3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < nout) orow32[n + e] = v[e];
+        }
+        return;
+      }
       unsigned short* orow = (unsigned short*)a.O + (long long)m * a.ldo;
       const bool vec_ok = ((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 7) == 0);
       if (vec_ok && n + 3 < nout) {

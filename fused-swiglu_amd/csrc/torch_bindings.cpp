@@ -4,7 +4,8 @@
 // `fused_swiglu_bf16(X, W1W3)` and `swiglu_fwd_bf16(m, n, k, A, ldA, B, ldB, C, ldC)`, the dispatcher library
 // `ASMLLM` with the same two schema strings, and the CUDA dispatch key (HIP tensors dispatch through it on
 // PyTorch-ROCm). Added beside them, because the full MLP forward and the fp16 configuration need them:
-// `fused_swiglu_fp16`, `swiglu_down_{bf16,fp16}`, `fused_swiglu_mlp_{bf16,fp16}`.
+// `fused_swiglu_fp16`, `swiglu_down_{bf16,fp16}`, `fused_swiglu_mlp_{bf16,fp16}`, and for the reference's build with
+// a float output type (constants.cuh:9-14) `fused_swiglu_bf16_f32out` and a float C in `swiglu_fwd_bf16`.
 //
 // This file is plain host C++ (no device code, no CUDA spellings): torch is used for tensors, the device guard
 // and the current stream only.
@@ -40,7 +41,11 @@ void swiglu_fwd_typed(at::ScalarType want, int64_t m, int64_t n, int64_t k, Tens
   // dtype guards as at swiglu.cu:475-480 (same failure mode: c10::Error -> RuntimeError)
   TORCH_CHECK(A.scalar_type() == want, "Expected tensor A to be of type ", want, ", but got: ", A.scalar_type());
   TORCH_CHECK(B.scalar_type() == want, "Expected tensor B to be of type ", want, ", but got: ", B.scalar_type());
-  TORCH_CHECK(C.scalar_type() == want, "Expected tensor C to be of type ", want, ", but got: ", C.scalar_type());
+  // C: the element type (the reference as shipped, C_TYPE bf16), or float: its other build (constants.cuh:9-14,
+  // "C can work with either bf16 or fp32", swiglu.cu:470-471), which stores the gated fp32 value unrounded
+  const bool c_f32 = C.scalar_type() == at::kFloat;
+  TORCH_CHECK(C.scalar_type() == want || c_f32, "Expected tensor C to be of type ", want, " or ", at::kFloat,
+              ", but got: ", C.scalar_type());
   check_device_tensor(A, "A");
   check_device_tensor(B, "B");
   check_device_tensor(C, "C");
@@ -54,8 +59,10 @@ void swiglu_fwd_typed(at::ScalarType want, int64_t m, int64_t n, int64_t k, Tens
   }
   const at::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(A));
   // like the reference's launcher this allocates nothing: the kernels read A and B where they lie
-  const int rc = fsw_gateup(dtype_code(want), m, n, k, A.data_ptr(), ldA, B.data_ptr(), ldB, C.data_ptr(), ldC / 2,
-                            current_stream());
+  const int rc = c_f32 ? fsw_gateup_f32out(dtype_code(want), m, n, k, A.data_ptr(), ldA, B.data_ptr(), ldB,
+                                           (float*)C.data_ptr(), ldC / 2, current_stream())
+                       : fsw_gateup(dtype_code(want), m, n, k, A.data_ptr(), ldA, B.data_ptr(), ldB, C.data_ptr(),
+                                    ldC / 2, current_stream());
   check_rc(rc, "swiglu_fwd");
 }
 
@@ -65,7 +72,7 @@ void swiglu_fwd_bf16(int64_t m, int64_t n, int64_t k, Tensor const& A, int64_t l
 }
 
 // fused_swiglu_bf16 of the reference (swiglu.cu:538-553): shapes from the tensors, out[M, N/2] with X's options.
-Tensor fused_swiglu_typed(at::ScalarType want, Tensor const& X, Tensor const& W1W3) {
+Tensor fused_swiglu_typed(at::ScalarType want, Tensor const& X, Tensor const& W1W3, bool f32_out = false) {
   TORCH_CHECK(X.dim() == 2 && W1W3.dim() == 2, "X and W1W3 must be 2-D");
   TORCH_CHECK(X.size(1) == W1W3.size(1), "X is [M, K] and W1W3 is [2*ff, K]: K differs (", X.size(1), " vs ",
               W1W3.size(1), ")");
@@ -73,7 +80,7 @@ Tensor fused_swiglu_typed(at::ScalarType want, Tensor const& X, Tensor const& W1
   TORCH_CHECK(W1W3.stride(1) == 1 || W1W3.size(1) <= 1, "W1W3 must be K-contiguous");
   const int64_t M = X.size(0), N = W1W3.size(0), K = X.size(1);
   TORCH_CHECK(N % 2 == 0, "W1W3 must hold an even number of rows (interleaved up/gate pairs)");
-  Tensor out = at::empty({M, N / 2}, X.options().dtype(want));
+  Tensor out = at::empty({M, N / 2}, X.options().dtype(f32_out ? at::kFloat : want));
   const int64_t ldx = M > 1 ? X.stride(0) : K;
   const int64_t ldw = N > 1 ? W1W3.stride(0) : K;
   swiglu_fwd_typed(want, M, N, K, X, ldx, W1W3, ldw, out, N);
@@ -82,6 +89,10 @@ Tensor fused_swiglu_typed(at::ScalarType want, Tensor const& X, Tensor const& W1
 
 Tensor fused_swiglu_bf16(Tensor const& X, Tensor const& W1W3) { return fused_swiglu_typed(at::kBFloat16, X, W1W3); }
 Tensor fused_swiglu_fp16(Tensor const& X, Tensor const& W1W3) { return fused_swiglu_typed(at::kHalf, X, W1W3); }
+// fused_swiglu_bf16 as the reference's C_TYPE float build returns it: float32, no rounding of the gated value
+Tensor fused_swiglu_bf16_f32out(Tensor const& X, Tensor const& W1W3) {
+  return fused_swiglu_typed(at::kBFloat16, X, W1W3, true);
+}
 
 // Y[M, D] = H[M, FF] @ W2[D, FF].T  (no counterpart in the reference)
 Tensor swiglu_down_typed(at::ScalarType want, Tensor const& H, Tensor const& W2) {
@@ -163,6 +174,9 @@ Tensor meta_down(at::ScalarType want, Tensor const& H, Tensor const& W2) {
 }
 Tensor meta_fused_swiglu_bf16(Tensor const& X, Tensor const& W) { return meta_gateup(at::kBFloat16, X, W); }
 Tensor meta_fused_swiglu_fp16(Tensor const& X, Tensor const& W) { return meta_gateup(at::kHalf, X, W); }
+Tensor meta_fused_swiglu_bf16_f32out(Tensor const& X, Tensor const& W) {
+  return meta_gateup(at::kBFloat16, X, W).to(at::kFloat);
+}
 Tensor meta_down_bf16(Tensor const& H, Tensor const& W2) { return meta_down(at::kBFloat16, H, W2); }
 Tensor meta_down_fp16(Tensor const& H, Tensor const& W2) { return meta_down(at::kHalf, H, W2); }
 Tensor meta_mlp_bf16(Tensor const& X, Tensor const& W, Tensor const& W2) {
@@ -180,6 +194,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("swiglu_fwd_bf16", &swiglu_fwd_bf16, "SwiGLU fwd bf16");
   // additions
   m.def("fused_swiglu_fp16", &fused_swiglu_fp16, "fused SwiGLU for fp16");
+  m.def("fused_swiglu_bf16_f32out", &fused_swiglu_bf16_f32out, "fused SwiGLU for bf16 inputs, float32 output");
   m.def("swiglu_down_bf16", &swiglu_down_bf16, "down projection H @ W2.T, bf16");
   m.def("swiglu_down_fp16", &swiglu_down_fp16, "down projection H @ W2.T, fp16");
   m.def("fused_swiglu_mlp_bf16", &fused_swiglu_mlp_bf16, "full SwiGLU MLP forward, bf16");
@@ -194,6 +209,7 @@ TORCH_LIBRARY(ASMLLM, m) {
   m.def("swiglu_fwd_bf16(int m, int n, int k, Tensor A, int ldA, Tensor B, int ldB, Tensor C, int ldC) -> ()");
   // additions
   m.def("fused_swiglu_fp16(Tensor X, Tensor W1W3) -> Tensor");
+  m.def("fused_swiglu_bf16_f32out(Tensor X, Tensor W1W3) -> Tensor");
   m.def("swiglu_down_bf16(Tensor H, Tensor W2) -> Tensor");
   m.def("swiglu_down_fp16(Tensor H, Tensor W2) -> Tensor");
   m.def("fused_swiglu_mlp_bf16(Tensor X, Tensor W1W3, Tensor W2) -> Tensor");
@@ -206,6 +222,7 @@ TORCH_LIBRARY_IMPL(ASMLLM, CUDA, m) {
   m.impl("fused_swiglu_bf16", &fused_swiglu_bf16);
   m.impl("swiglu_fwd_bf16", &swiglu_fwd_bf16);
   m.impl("fused_swiglu_fp16", &fused_swiglu_fp16);
+  m.impl("fused_swiglu_bf16_f32out", &fused_swiglu_bf16_f32out);
   m.impl("swiglu_down_bf16", &swiglu_down_bf16);
   m.impl("swiglu_down_fp16", &swiglu_down_fp16);
   m.impl("fused_swiglu_mlp_bf16", &fused_swiglu_mlp_bf16);
@@ -216,6 +233,7 @@ TORCH_LIBRARY_IMPL(ASMLLM, CUDA, m) {
 TORCH_LIBRARY_IMPL(ASMLLM, Meta, m) {
   m.impl("fused_swiglu_bf16", &meta_fused_swiglu_bf16);
   m.impl("fused_swiglu_fp16", &meta_fused_swiglu_fp16);
+  m.impl("fused_swiglu_bf16_f32out", &meta_fused_swiglu_bf16_f32out);
   m.impl("swiglu_down_bf16", &meta_down_bf16);
   m.impl("swiglu_down_fp16", &meta_down_fp16);
   m.impl("fused_swiglu_mlp_bf16", &meta_mlp_bf16);

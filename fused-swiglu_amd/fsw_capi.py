@@ -19,6 +19,7 @@ _i, _i64, _vp, _sz, _cp = ctypes.c_int, ctypes.c_int64, ctypes.c_void_p, ctypes.
 PROTOTYPES = {
     "fsw_validate_gateup": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "fsw_gateup": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "fsw_gateup_f32out": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "fsw_validate_down": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64]),
     "fsw_down_workspace_bytes": (_sz, [_i, _i64, _i64, _i64]),
     "fsw_down": (_i, [_i, _i64, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _sz, _vp]),
@@ -145,11 +146,31 @@ def gateup(X, W13, out=None):
     if out is None:
         out = torch.empty((M, N // 2), dtype=X.dtype, device=X.device)
     _check_operands(X, out=out, out_shape=(M, N // 2))
-    nbytes = lib().fsw_gateup_workspace_bytes(code, M, N, K)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device) if nbytes else None
     with torch.cuda.device(X.device):
-        check(lib().fsw_gateup_ws(code, M, N, K, X.data_ptr(), _ld(X), W13.data_ptr(), _ld(W13), out.data_ptr(),
-                                  _ld(out), ws.data_ptr() if ws is not None else None, nbytes, _stream(X)))
+        check(lib().fsw_gateup(code, M, N, K, X.data_ptr(), _ld(X), W13.data_ptr(), _ld(W13), out.data_ptr(),
+                               _ld(out), _stream(X)))
+    return out
+
+
+def gateup_f32out(X, W13, out=None):
+    """H[M, ff] as float32, the gated fp32 value unrounded, through fsw_gateup_f32out."""
+    import torch
+    code = dtype_code(X)
+    if W13.dtype != X.dtype:
+        raise FswError(E_DTYPE, "fsw: X and W13 differ in element type")
+    _check_operands(X, W13)
+    M, K = X.shape
+    N = W13.shape[0]
+    if W13.shape[1] != K:
+        raise FswError(E_SHAPE, "fsw: X is [M, K] and W13 is [2 ff, K]: K differs")
+    if out is None:
+        out = torch.empty((M, N // 2), dtype=torch.float32, device=X.device)
+    if out.dtype != torch.float32 or tuple(out.shape) != (M, N // 2):
+        raise FswError(E_SHAPE, "fsw: `out` must be a float32 tensor of shape %s" % ((M, N // 2),))
+    _check_operands(out)
+    with torch.cuda.device(X.device):
+        check(lib().fsw_gateup_f32out(code, M, N, K, X.data_ptr(), _ld(X), W13.data_ptr(), _ld(W13), out.data_ptr(),
+                                      _ld(out), _stream(X)))
     return out
 
 

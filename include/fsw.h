@@ -76,6 +76,16 @@ FSW_API int fsw_gateup(int dtype, int64_t M, int64_t N, int64_t K,
                const void* X, int64_t ldx, const void* W13, int64_t ldw,
                void* H, int64_t ldh, void* stream);
 
+/*
+ * fsw_gateup whose H is float [M, N/2] (row stride ldh in floats, 4-byte aligned): the gated fp32 value is stored
+ * as it is, with no rounding. Replaces swiglu_fwd<bf16,bf16,float>, the reference's build with C_TYPE float
+ * (constants.cuh:9-14; cast_mmaresult's to_float branch, swiglu.cu:47-82; "C can work with either bf16 or fp32",
+ * swiglu.cu:470-471). Inputs as for fsw_gateup.
+ */
+FSW_API int fsw_gateup_f32out(int dtype, int64_t M, int64_t N, int64_t K,
+                      const void* X, int64_t ldx, const void* W13, int64_t ldw,
+                      float* H, int64_t ldh, void* stream);
+
 /* Host-only validation of fsw_down: M, D, FF >= 0; FF % 8 == 0; ldh >= FF, ldw2 >= FF, ldy >= D;
  * ldh % 8 == 0, ldw2 % 8 == 0; H, W2 16-byte aligned. */
 FSW_API int fsw_validate_down(int dtype, int64_t M, int64_t D, int64_t FF,

@@ -534,6 +534,57 @@ def test_swiglu_fwd_bf16_writes_dense_half_width_rows(ext):
         ext.swiglu_fwd_bf16(M, N + 1, K, g["X"], K, g["W13"], K, C, N)  # odd N
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [1, 16, 64, 65, 300, 1024])
+def test_float32_output_is_the_unrounded_gated_value(capi, M, dtype):
+    """fsw_gateup_f32out (the reference's build with C_TYPE float, constants.cuh:9-14, swiglu.cu:470-471): H in
+    float32 is up * silu(gate) to fp32 accumulation noise, three orders below a 16-bit rounding; rounding it once gives
+    the 16-bit kernel's output bit for bit (same kernel, same K order: the 16-bit path rounds exactly this value)."""
+    for (d, ff) in [(512, 1032), (1000, 264), (64, 40)]:
+        inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=5 * M + d, x_scale=0.5)
+        g = to_dev(inp)
+        H32 = capi.gateup_f32out(g["X"], g["W13"])
+        assert H32.dtype == torch.float32 and tuple(H32.shape) == (M, ff)
+        ref = oracle.ref_gateup(inp["X"], inp["W13"], torch.float64)
+        err = (H32.cpu().double() - ref).abs()
+        assert not (err > 1e-5 * (1.0 + ref.abs())).any(), "fp32 H %s: worst |d| = %g" % ((M, d, ff), err.max().item())
+        try:
+            capi.set_variant(0, 100 if M <= 64 else 5)  # the kernel the fp32 path runs for this M
+            H16 = capi.gateup(g["X"], g["W13"])
+        finally:
+            capi.set_variant(0, -1)
+        assert torch.equal(H16, H32.to(dtype))
+    # strided float output inside a wider NaN buffer, odd row stride (scalar stores): neighbours untouched
+    d, ff = 512, 1032
+    inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=77, x_scale=0.5)
+    g = to_dev(inp)
+    wide = torch.full((M, ff + 5), float("nan"), dtype=torch.float32, device=DEV)
+    capi.gateup_f32out(g["X"], g["W13"], out=wide[:, :ff])
+    assert torch.equal(wide[:, :ff], capi.gateup_f32out(g["X"], g["W13"])) and torch.isnan(wide[:, ff:]).all()
+
+
+def test_float32_output_through_the_operators(ext):
+    """fused_swiglu_bf16_f32out, and swiglu_fwd_bf16 with a float C (the reference's operator compiled with C_TYPE
+    float): the ldC / 2 rule holds in elements of C's type (swiglu.cu:414); wrong C types still raise."""
+    M, K, N = 300, 512, 2064
+    g = torch.Generator(device=DEV).manual_seed(31)
+    X = (torch.randn((M, K), device=DEV, generator=g) * 0.5).to(torch.bfloat16)
+    W = (torch.randn((N, K), device=DEV, generator=g) / K ** 0.5).to(torch.bfloat16)
+    H32 = ext.fused_swiglu_bf16_f32out(X, W)
+    assert H32.dtype == torch.float32 and tuple(H32.shape) == (M, N // 2)
+    ref = oracle.ref_gateup(X.cpu(), W.cpu(), torch.float64)
+    assert ((H32.cpu().double() - ref).abs() <= 1e-5 * (1.0 + ref.abs())).all()
+    assert torch.equal(torch.ops.ASMLLM.fused_swiglu_bf16_f32out(X, W), H32)
+    C = torch.full((M, N), float("nan"), device=DEV, dtype=torch.float32)
+    ext.swiglu_fwd_bf16(M, N, K, X, K, W, K, C, N)
+    flat = C.view(-1)
+    assert torch.equal(flat[: M * (N // 2)].view(M, N // 2), H32) and torch.isnan(flat[M * (N // 2):]).all()
+    with pytest.raises(RuntimeError):
+        ext.swiglu_fwd_bf16(M, N, K, X, K, W, K, torch.empty((M, N), device=DEV, dtype=torch.float16), N)
+    with pytest.raises(RuntimeError):
+        ext.swiglu_fwd_bf16(M, N, K, X, K, W, K, torch.empty((M, N), device=DEV, dtype=torch.float64), N)
+
+
 def test_strided_views_and_row_independence(capi):
     inp = fsw_weights.make_inputs(150, 192, 144, torch.bfloat16, seed=36)
     g = to_dev(inp)
