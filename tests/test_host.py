@@ -262,7 +262,8 @@ def test_wrong_dtype_raises_runtime_error_like_the_reference(ext):
     with pytest.raises(RuntimeError, match="Expected tensor B to be of type"):
         ext.swiglu_fwd_bf16(4, 6, 8, X32.bfloat16(), 8, W32, 8, torch.zeros(4, 6, dtype=torch.bfloat16), 6)
     with pytest.raises(RuntimeError, match="Expected tensor C to be of type"):
-        ext.swiglu_fwd_bf16(4, 6, 8, X32.bfloat16(), 8, W32.bfloat16(), 8, torch.zeros(4, 6), 6)
+        # float32 is the reference's other output type (constants.cuh:9-14) and is accepted; float16 is not
+        ext.swiglu_fwd_bf16(4, 6, 8, X32.bfloat16(), 8, W32.bfloat16(), 8, torch.zeros(4, 6, dtype=torch.float16), 6)
     # CPU tensors of the right dtype are refused (no CPU fallback exists)
     with pytest.raises(RuntimeError, match="GPU"):
         ext.fused_swiglu_bf16(X32.bfloat16(), W32.bfloat16())
