@@ -17,7 +17,7 @@ Extra objects on the same line:
                  512 MiB cache-defeating write before every timed call): median / p20 / p80 and roofline fraction;
   comparator   — the vendor GEMM (torch.mm, hipBLASLt) on the gate/up and down shapes of the workload, same run;
   ceilings     — what this board sustains with nothing in the way: a register-only MFMA loop with random operands
-                 and a plain streaming read (fsw_probe_mfma / fsw_probe_read);
+                 and a plain streaming read (fsw_probe_mfma / fsw_probe_read of libfsw_probe.so);
   decode       — the M=16 weight-streaming configuration in GB/s against the HBM3E peak: `value` in steady state on
                  one set of weights, `cold` alternating three copies of the weights (1.06 GB, beyond every cache);
   cpu_baseline — the same formulation in fp32 PyTorch on this host's cores (oracle/, the checker): whole forwards
@@ -286,8 +286,9 @@ def comparator_leg(torch, g, cfg, fsw_weights, steps, warmup, settle_ms):
 
 
 def ceilings_leg(capi, torch):
-    """Register-only MFMA loop (random bf16 operands) and a plain streaming read, through the library's probes."""
-    L = capi.lib()
+    """Register-only MFMA loop (random bf16 operands) and a plain streaming read, through the measurement
+    kernels of libfsw_probe.so (include/fsw_probe.h)."""
+    L = capi.probe_lib()
     stream = torch.cuda.current_stream().cuda_stream
     ops = torch.randn(8192, device="cuda:0").to(torch.bfloat16)          # 16 KB of N(0,1) operands
     outb = torch.empty(256 * 256, dtype=torch.float32, device="cuda:0")

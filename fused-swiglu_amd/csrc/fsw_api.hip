@@ -2,6 +2,7 @@
 // Replaces the host launcher swiglu_fwd<TA,TB,TC> (swiglu.cu:397-525) and the convenience op's shape
 // derivation (swiglu.cu:538-553); the public contract is include/fsw.h.
 #include <hip/hip_runtime.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <atomic>
@@ -177,6 +178,12 @@ int fsw_decode_barrier_failures(void) {
 
 int fsw_set_variant(int family, int variant) {
   if (family < 0 || family > 1) return FSW_E_VARIANT;
+  // the barrier that cannot complete exists for the failure-path test only: refused unless the process's
+  // environment holds FSW_TEST_HOOKS=1, so a caller cannot leave it set by accident and get forwards without Y
+  if (variant == VARIANT_DECODE_FUSED_FAIL) {
+    const char* hooks = getenv("FSW_TEST_HOOKS");
+    if (!hooks || strcmp(hooks, "1") != 0) return FSW_E_VARIANT;
+  }
   if (variant >= 0 && variant != VARIANT_SKINNY && variant != VARIANT_DECODE_STREAM &&
       !(family == 0 && (variant == VARIANT_DECODE_FUSED || variant == VARIANT_DECODE_FUSED_FAIL)) &&
       !(family == 1 && variant == VARIANT_STREAM_SPLIT) &&

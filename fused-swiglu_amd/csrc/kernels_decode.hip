@@ -30,9 +30,12 @@
 // zero by the last workgroup to depart). The host hands every single-launch forward a slot of its own and reuses a
 // slot only when the event recorded behind its previous launch has completed; with no free slot, or on a stream
 // that is being captured, the caller runs the two-launch path instead. The spin is bounded: if the workgroups are
-// not all resident (someone else holds CUs) a workgroup gives up, sets the slot's `failed` word and SKIPS the down
-// projection, as does every workgroup that sees the word set after the barrier: a failed launch leaves Y
-// incomplete and is reported by decode_barrier_failures(), it never hangs and never multiplies a partial H.
+// not all resident (someone else holds CUs) a workgroup gives up, writes the launch's own number (its epoch, unique
+// per device) into the slot's `failed` word and SKIPS the down projection, as does every workgroup that reads its
+// own epoch there after the barrier: a failed launch leaves Y incomplete and is counted in the slot's fourth word,
+// which decode_barrier_failures() reports and clears; it never hangs and never multiplies a partial H. The mark
+// belongs to the launch: a later launch that is handed the same slot carries another epoch and is not affected by
+// a failure nobody has asked about yet.
 #include <mutex>
 
 #include "fsw_internal.h"
@@ -47,7 +50,7 @@ constexpr int DEC_PF2 = 4;           // phase 2: weight steps in flight per wave
 constexpr int DEC_POLL_SLEEP = 8;    // s_sleep between polls: 256 pollers must not saturate the counter's channel
 constexpr int DEC_SLOTS = 64;        // barrier slots for launches in flight at the same time
 constexpr unsigned DEC_SPIN_LIMIT = 1u << 18;  // ~0.3 s of polling
-static __device__ unsigned g_dec_barrier[DEC_SLOTS * 4];  // per slot: arrive, depart, failed, pad
+static __device__ unsigned g_dec_barrier[DEC_SLOTS * 4];  // per slot: arrive, depart, epoch of a failed launch, failures
 
 // phases: bit 0 = gate/up, bit 1 = down; 3 = both with the device-wide barrier in between, which waits until
 // `expected` workgroups have arrived (the grid size; a test passes more, so that the bounded wait gives up) for at
@@ -55,7 +58,7 @@ static __device__ unsigned g_dec_barrier[DEC_SLOTS * 4];  // per slot: arrive, d
 template <class E>
 __global__ void __launch_bounds__(DEC_NW * 64)
 decode_mlp_kernel(const DecodeArgs a, unsigned* bar, const int phases, const unsigned expected,
-                  const unsigned spin_limit) {
+                  const unsigned spin_limit, const unsigned epoch) {
   constexpr int KS = 128;
   // slabs of the waves first; the phase-1 reduction reuses everything, the phase-2 reduction has its own two
   // buffers behind the slabs
@@ -265,14 +268,16 @@ decode_mlp_kernel(const DecodeArgs a, unsigned* bar, const int phases, const uns
       unsigned spins = 0, failed = 0;
       while (__hip_atomic_load(bar + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < expected) {
         if (++spins > spin_limit) {  // not all workgroups are resident: give up rather than hang
-          __hip_atomic_store(bar + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          // mark the slot with this launch's epoch; the workgroup that changes the word counts the failure once
+          if (__hip_atomic_exchange(bar + 2, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != epoch)
+            __hip_atomic_fetch_add(bar + 3, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           failed = 1;
           break;
         }
         __builtin_amdgcn_s_sleep(DEC_POLL_SLEEP);
       }
       // a workgroup that got through still skips the down projection when another one has given up
-      if (!failed) failed = __hip_atomic_load(bar + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (!failed) failed = __hip_atomic_load(bar + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == epoch ? 1u : 0u;
       barrier_failed = failed;
       // depart: the last workgroup out restores the slot for the next launch that is handed it
       const unsigned left = __hip_atomic_fetch_add(bar + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -375,6 +380,7 @@ struct DecodeDevice {
   hipEvent_t done[DEC_SLOTS] = {};   // recorded behind the last launch that used the slot
   bool used[DEC_SLOTS] = {};
   unsigned next = 0;
+  unsigned epoch = 0;                // number of the last single-launch forward on this device (never 0 in use)
 };
 std::mutex g_dec_mutex;
 DecodeDevice g_dec_dev[64];
@@ -441,14 +447,19 @@ hipError_t launch_decode_mlp(int dtype, const DecodeArgs& a, hipStream_t stream,
     d->next = (unsigned)slot + 1;
   }
   unsigned* bar = d->bar + (slot < 0 ? 0 : slot) * 4;
+  unsigned epoch = 0;
+  if (slot >= 0) {
+    if (++d->epoch == 0) ++d->epoch;  // 0 is what an untouched slot holds
+    epoch = d->epoch;
+  }
   const unsigned expected = (unsigned)grid + (test_unreachable ? 1u : 0u);
   const unsigned spin_limit = test_unreachable ? 64u : DEC_SPIN_LIMIT;
   if (dtype == 0) {
     hipLaunchKernelGGL((decode_mlp_kernel<Bf16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar, phases,
-                       expected, spin_limit);
+                       expected, spin_limit, epoch);
   } else {
     hipLaunchKernelGGL((decode_mlp_kernel<Fp16>), dim3((unsigned)grid), dim3(DEC_NW * 64), 0, stream, a, bar, phases,
-                       expected, spin_limit);
+                       expected, spin_limit, epoch);
   }
   e = hipGetLastError();
   if (e != hipSuccess) return e;
@@ -470,9 +481,9 @@ hipError_t decode_barrier_failures(int* count) {
   if (e != hipSuccess) return e;
   const unsigned zero = 0;
   for (int s = 0; s < DEC_SLOTS; ++s) {
-    if (host[s * 4 + 2] == 0) continue;
-    ++*count;
-    e = hipMemcpy(d->bar + s * 4 + 2, &zero, sizeof(zero), hipMemcpyHostToDevice);
+    if (host[s * 4 + 3] == 0) continue;
+    *count += (int)host[s * 4 + 3];
+    e = hipMemcpy(d->bar + s * 4 + 3, &zero, sizeof(zero), hipMemcpyHostToDevice);
     if (e != hipSuccess) return e;
   }
   return hipSuccess;

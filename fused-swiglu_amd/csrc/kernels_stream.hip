@@ -188,7 +188,16 @@ stream_split_kernel(const GemmArgs a, float* __restrict__ part, unsigned* __rest
                              __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    // every partial of this workgroup has been acknowledged by memory before the ticket is drawn
+    // every partial of this workgroup has been acknowledged by memory before the ticket is drawn.
+    // The ordering between workgroups rests on three facts of this target, not on language-level fences: (i) the
+    // agent-scope atomic stores above are written through to memory, and vmcnt reaches zero only when memory has
+    // acknowledged them, so the ticket drawn below follows the partials; (ii) the agent-scope atomic loads of the
+    // last workgroup are served by memory, never by a stale line of its own XCD's L2; (iii) a wave's memory
+    // instructions issue in program order, and those loads sit behind the branch on the ticket. A release fence
+    // and an acquire fence at agent scope would say the same in the language, but on this target they write the
+    // whole L2 back and invalidate it: measured on a kernel of this family at 4096 x 14336, 23 -> 60 us. A later edit
+    // that turns a partial store or load into a plain access breaks (i) or (ii) silently across the XCDs' L2s; the
+    // bit-equality of repeated calls in the tests is what would show it.
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if (t == 0) {
       const unsigned ticket = __hip_atomic_fetch_add(tickets + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

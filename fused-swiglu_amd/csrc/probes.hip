@@ -1,11 +1,14 @@
-// Two measurement kernels behind the C ABI (fsw_probe_mfma, fsw_probe_read): what the matrix pipes and the memory
-// system of THIS board sustain with nothing else in the way, measured in the same process as the product kernels.
+// Two measurement kernels in a library of their own (libfsw_probe.so, include/fsw_probe.h; not part of the product
+// library): what the matrix pipes and the memory system of THIS board sustain with nothing else in the way, measured
+// in the same process as the product kernels.
 // They are the yardsticks bench.py prints beside the roofline fractions (the published peaks assume a clock the
 // board does not hold under a full MFMA load with random operands, and a read stream never sees the pin bandwidth).
 // No counterpart in the reference.
 #include <hip/hip_runtime.h>
+#include <string.h>
 
-#include "fsw.h"
+#include "fsw.h"  // error codes only
+#include "fsw_probe.h"
 #include "fsw_device.h"
 
 namespace fsw {
@@ -63,6 +66,16 @@ __global__ void __launch_bounds__(256) probe_read_kernel(const u32x4* __restrict
 
 }  // namespace fsw
 
+namespace {
+// the kernels are gfx950 code: anything else is refused before a launch
+bool on_gfx950() {
+  int dev = 0;
+  hipDeviceProp_t prop;
+  if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return false;
+  return strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+}
+}  // namespace
+
 extern "C" {
 
 int fsw_probe_mfma(int dtype, int iters, const void* operands, void* out, int workgroups, void* stream) {
@@ -70,6 +83,7 @@ int fsw_probe_mfma(int dtype, int iters, const void* operands, void* out, int wo
   if (iters < 0 || workgroups < 1 || workgroups > 65536) return FSW_E_SHAPE;
   if (!operands || !out) return FSW_E_NULL;
   if (((uintptr_t)operands) & 15) return FSW_E_ALIGN;
+  if (!on_gfx950()) return FSW_E_DEVICE;
   if (dtype == FSW_BF16) {
     hipLaunchKernelGGL((fsw::probe_mfma_kernel<fsw::Bf16>), dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream,
                        (const fsw::u32x4*)operands, (float*)out, iters);
@@ -84,6 +98,7 @@ int fsw_probe_read(const void* src, size_t bytes, void* out, int workgroups, voi
   if (!src || !out) return FSW_E_NULL;
   if ((((uintptr_t)src) & 15) || (bytes & 15)) return FSW_E_ALIGN;
   if (workgroups < 1 || workgroups > 65536) return FSW_E_SHAPE;
+  if (!on_gfx950()) return FSW_E_DEVICE;
   hipLaunchKernelGGL(fsw::probe_read_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream,
                      (const fsw::u32x4*)src, bytes / 16, (unsigned*)out);
   return hipGetLastError() == hipSuccess ? FSW_OK : FSW_E_LAUNCH;

@@ -40,13 +40,19 @@ PROTOTYPES = {
     "fsw_last_hip_error": (_i, []),
     "fsw_decode_barrier_failures": (_i, []),
     "fsw_version": (_i, []),
-    "fsw_probe_mfma": (_i, [_i, _i, _vp, _vp, _i, _vp]),
-    "fsw_probe_read": (_i, [_vp, _sz, _vp, _i, _vp]),
     "fsw_set_variant": (_i, [_i, _i]),
     "fsw_variant_name": (_cp, [_i, _i, _i64, _i64, _i64]),
 }
 
+# the benchmark's measurement kernels live in a library of their own (include/fsw_probe.h)
+PROBE_LIB_PATH = os.path.join(HERE, "libfsw_probe.so")
+PROBE_PROTOTYPES = {
+    "fsw_probe_mfma": (_i, [_i, _i, _vp, _vp, _i, _vp]),
+    "fsw_probe_read": (_i, [_vp, _sz, _vp, _i, _vp]),
+}
+
 _lib = None
+_probe_lib = None
 
 
 class FswError(RuntimeError):
@@ -75,6 +81,21 @@ def lib():
             fn.restype, fn.argtypes = res, args
         _lib = L
     return _lib
+
+
+def probe_lib():
+    """libfsw_probe.so (measurement kernels for bench.py), loaded after the product library."""
+    global _probe_lib
+    if _probe_lib is None:
+        lib()
+        if not os.path.exists(PROBE_LIB_PATH):
+            raise FileNotFoundError("%s is missing: build it with `python setup.py build_hip` in %s" % (PROBE_LIB_PATH, HERE))
+        L = ctypes.CDLL(PROBE_LIB_PATH)
+        for name, (res, args) in PROBE_PROTOTYPES.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _probe_lib = L
+    return _probe_lib
 
 
 def strerror(code):

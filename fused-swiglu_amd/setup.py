@@ -3,7 +3,8 @@
 Counterpart of the reference's setup.py:12-45 (CUDAExtension + nvcc sm_80), in two steps:
 
   1. the HIP kernels and the C-ABI dispatcher (csrc/*.hip) are compiled by hipcc for gfx950 into
-     `libfsw_hip.so`, which exports only the C symbols declared in include/fsw.h;
+     `libfsw_hip.so`, which exports only the C symbols declared in include/fsw.h (and the benchmark's two
+     measurement kernels, csrc/probes.hip, into `libfsw_probe.so`, include/fsw_probe.h);
   2. csrc/torch_bindings.cpp is built as a host-only C++ extension (`CppExtension`, so torch's source
      translation pass for CUDA extensions never runs) that links `libfsw_hip.so`.
 
@@ -20,7 +21,9 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 OBJ_DIR = os.path.join(HERE, "build", "hip_obj")
 LIB_NAME = "libfsw_hip.so"
-HIP_SOURCES = ["kernels_pair16.hip", "kernels_tiled.hip", "kernels_skinny.hip", "kernels_stream.hip", "kernels_decode.hip", "probes.hip", "fsw_api.hip"]
+HIP_SOURCES = ["kernels_pair16.hip", "kernels_tiled.hip", "kernels_skinny.hip", "kernels_stream.hip", "kernels_decode.hip", "fsw_api.hip"]
+PROBE_LIB_NAME = "libfsw_probe.so"  # measurement kernels of the benchmark (include/fsw_probe.h): not part of the product
+PROBE_SOURCES = ["probes.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -33,7 +36,7 @@ HIP_FLAGS = [
 def build_hip(verbose=True):
     """Compile csrc/*.hip for gfx950 and link libfsw_hip.so next to this file. Always recompiles."""
     os.makedirs(OBJ_DIR, exist_ok=True)
-    sources = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    sources = [s for s in HIP_SOURCES + PROBE_SOURCES if os.path.exists(os.path.join(CSRC, s))]
 
     def compile_one(src):
         obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
@@ -51,10 +54,12 @@ def build_hip(verbose=True):
     with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
         objs = list(pool.map(compile_one, sources))
     lib = os.path.join(HERE, LIB_NAME)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
+    probe_objs = [o for o in objs if os.path.basename(o).replace(".o", ".hip") in PROBE_SOURCES]
+    for out, members in ((lib, [o for o in objs if o not in probe_objs]), (os.path.join(HERE, PROBE_LIB_NAME), probe_objs)):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + members
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True)
     return lib
 
 

@@ -191,7 +191,10 @@ FSW_API int fsw_version(void);
  * for M <= 64; the dispatcher itself picks it up to 16 .. 48 rows, the larger the weights the fewer); 102 is the
  * persistent streaming kernel (honoured for M <= 16; automatic only for d * ff >= 2^27); family 0 variant 101
  * makes fsw_mlp run M <= 16 as ONE persistent launch (gate/up, device-wide barrier, down) instead of two launches
- * -- see fsw_decode_barrier_failures(); 103 is 101 with a barrier that cannot complete (failure-path test);
+ * -- see fsw_decode_barrier_failures(): a correctness-tested experiment that measures SLOWER than the two launches
+ * (69.7 vs 61.0 us at M = 16, d = 4096, ff = 14336) and is kept for study only; 103 is 101 with a barrier that cannot
+ * complete, a hook of the failure-path test that is refused (FSW_E_VARIANT) unless the environment holds
+ * FSW_TEST_HOOKS=1;
  * family 1 variant 104 makes fsw_mlp run the down projection of M <= 32 rows on the split-K streaming kernel
  * (32-row tiles, two K ranges whose partial tiles meet through ticket counters that the gate/up kernel zeroes)
  * whatever the shape; the dispatcher picks it for 17 .. 32 rows of large weight matrices.
@@ -210,17 +213,6 @@ FSW_API int fsw_set_variant(int family, int variant);
  * two-launch path instead. No counterpart in the reference.
  */
 FSW_API int fsw_decode_barrier_failures(void);
-
-/*
- * Measurement kernels (no counterpart in the reference): what this board sustains with nothing else in the way,
- * for the benchmark to print beside its roofline fractions.
- * fsw_probe_mfma: `workgroups` x 4 waves each issue iters x 64 v_mfma_f32_16x16x32 from registers (the prefill
- *   kernel's accumulator shape); = workgroups * 4 * iters * 64 * 16384 FLOP. `operands`: 16 KB of device data in the
- *   element type (its values set the power draw), 16-byte aligned; `out`: workgroups * 1 KB of device scratch.
- * fsw_probe_read: streams `bytes` (a multiple of 16) from `src` once with non-temporal 16-byte loads; `out`: 4 bytes.
- */
-FSW_API int fsw_probe_mfma(int dtype, int iters, const void* operands, void* out, int workgroups, void* stream);
-FSW_API int fsw_probe_read(const void* src, size_t bytes, void* out, int workgroups, void* stream);
 
 /* Name of the kernel variant the dispatcher picks for this shape (static storage); "splitk_<kernel>" when the
  * down projection splits K (family 1; K_or_FF decides). family 2: the down projection as fsw_mlp runs it (differs

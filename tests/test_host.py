@@ -31,6 +31,18 @@ def test_library_exports_every_declared_symbol(capi):
     assert capi.lib().fsw_version() >= 1000
 
 
+def test_probe_library_is_separate_from_the_product(capi):
+    """The benchmark's measurement kernels are not part of the product ABI: their own header, their own library."""
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "fsw_probe.h")).read(), flags=re.S)
+    names = re.findall(r"FSW_PROBE_API\s+[\w\s\*]+?\b(fsw_\w+)\s*\(", text)
+    assert sorted(names) == sorted(capi.PROBE_PROTOTYPES) == ["fsw_probe_mfma", "fsw_probe_read"]
+    probe = ctypes.CDLL(capi.PROBE_LIB_PATH)
+    product = ctypes.CDLL(capi.LIB_PATH)
+    for n in names:
+        assert hasattr(probe, n) and not hasattr(product, n)
+    assert "fsw_probe" not in open(HEADER).read()
+
+
 def test_strerror_covers_all_codes(capi):
     seen = set()
     for code in range(0, -11, -1):

@@ -276,15 +276,42 @@ def test_single_launch_decode_reports_a_failed_barrier(capi):
     torch.cuda.synchronize()
     assert capi.decode_barrier_failures() == 0
     Y = torch.full((M, d), 7.0, dtype=torch.bfloat16, device=DEV)
-    try:
-        capi.set_variant(0, 103)
-        capi.mlp(g["X"], g["W13"], g["W2"], out=Y, workspace=ws)
-        torch.cuda.synchronize()
-    finally:
-        capi.set_variant(0, -1)
-    assert (Y.float() == 7.0).all(), "a failed single launch must not write Y"
+    # the failing barrier is a test hook: refused unless the process asks for test hooks
+    os.environ.pop("FSW_TEST_HOOKS", None)
+    assert capi.lib().fsw_set_variant(0, 103) == capi.E_VARIANT
+    os.environ["FSW_TEST_HOOKS"] = "1"
+
+    def failing_launch():
+        Y.fill_(7.0)
+        try:
+            capi.set_variant(0, 103)
+            capi.mlp(g["X"], g["W13"], g["W2"], out=Y, workspace=ws)
+            torch.cuda.synchronize()
+        finally:
+            capi.set_variant(0, -1)
+        assert (Y.float() == 7.0).all(), "a failed single launch must not write Y"
+
+    failing_launch()
     assert capi.decode_barrier_failures() == 1
     assert capi.decode_barrier_failures() == 0
+    # the mark of a failure belongs to its launch: with nobody asking in between, 70 good launches (they walk over
+    # all 64 barrier slots, the failed one included) each write the whole of Y, and the failure is still reported
+    failing_launch()
+    good = capi.mlp(g["X"], g["W13"], g["W2"])
+    try:
+        capi.set_variant(0, 101)
+        for i in range(70):
+            Y.fill_(7.0)
+            capi.mlp(g["X"], g["W13"], g["W2"], out=Y, workspace=ws)
+            assert (Y.float() - good.float()).abs().max().item() <= 2e-2, "launch %d after an unreported failure" % i
+    finally:
+        capi.set_variant(0, -1)
+    assert capi.decode_barrier_failures() == 1
+    assert capi.decode_barrier_failures() == 0
+    failing_launch()
+    failing_launch()
+    assert capi.decode_barrier_failures() == 2
+    os.environ.pop("FSW_TEST_HOOKS", None)
     # the gate/up half did run, and the slot works again: 70 good launches walk over all 64 slots
     H = ws[: M * ff * 2].view(torch.bfloat16).view(M, ff)
     assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), torch.bfloat16, "H of a failed launch")
@@ -353,6 +380,20 @@ def test_split_k_streaming_down_inside_mlp(capi, M, dtype):
     assert name(17, 4096, 14336) == "stream_split" and name(32, 4096, 14336) == "stream_split"
     assert name(16, 4096, 14336) == "skinny" and name(24, 512, 1024) == "skinny" and name(33, 4096, 14336) != "stream_split"
     assert name(16, 8192, 28672) == "decode_stream"
+    # decode size with a ragged last tile (d % 32 != 0: 129 tiles, the last one 8 rows wide) and a K that the two
+    # workgroups of a tile and their waves do not split evenly
+    if M in (17, 32):
+        d, ff = 4104, 14344
+        assert name(M, d, ff) == "stream_split"
+        inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=8, x_scale=0.5)
+        g = to_dev(inp)
+        ws = capi.mlp_workspace(g["X"], ff)
+        ws.fill_(0xA5)
+        Y = capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws)
+        H = ws[: M * ff * 2].view(dtype).view(M, ff).clone()
+        assert_one_rounding(Y, oracle.ref_down(H.cpu(), inp["W2"], torch.float64), dtype, "stream-split ragged decode size")
+        for _ in range(5):
+            assert torch.equal(capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws), Y)
     if M in (17, 32):
         d, ff = 4096, 14336
         inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=7, x_scale=0.5)
