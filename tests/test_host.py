@@ -104,6 +104,26 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu(capi):
     assert L.fsw_mlp_workspace_bytes(0, 4, 16, 8) >= 4 * 8 * 2
     assert L.fsw_mlp_workspace_bytes(0, 0, 16, 8) == 0
     assert L.fsw_set_variant(0, 12345) == capi.E_VARIANT
+    # the float-output form of the gate/up product: the same rules, plus a 4-byte aligned H
+    f32 = L.fsw_gateup_f32out
+    assert f32(0, 4, 7, 16, 0x1000, 16, 0x2000, 16, 0x3000, 4, None) == capi.E_SHAPE
+    assert f32(2, 4, 8, 16, 0x1000, 16, 0x2000, 16, 0x3000, 4, None) == capi.E_DTYPE
+    assert f32(0, 4, 8, 16, 0x1000, 16, 0x2000, 16, 0x3000, 3, None) == capi.E_LD
+    assert f32(0, 4, 8, 16, 0x1000, 16, 0x2000, 16, 0x3002, 4, None) == capi.E_ALIGN
+    assert f32(0, 4, 8, 16, 0x1000, 16, 0x2000, 16, None, 4, None) == capi.E_NULL
+    assert f32(0, 0, 8, 16, None, 16, None, 16, None, 4, None) == capi.OK
+    # row-major X -> blocked H: as fsw_gateup, a K of zero has no blocked representation, H 16-byte aligned
+    hb = L.fsw_gateup_hblocked
+    assert hb(0, 4, 8, 12, 0x1000, 16, 0x2000, 16, 0, 0x3000, None) == capi.E_ALIGN
+    assert hb(0, 4, 8, 16, 0x1000, 8, 0x2000, 16, 0, 0x3000, None) == capi.E_LD
+    assert hb(0, 4, 8, 0, 0x1000, 16, 0x2000, 16, 0, 0x3000, None) == capi.E_SHAPE
+    assert hb(0, 4, 8, 16, 0x1000, 16, 0x2000, 16, 0, 0x3008, None) == capi.E_ALIGN
+    assert hb(0, 4, 8, 16, 0x1000, 16, 0x2000, 0, 1, None, None) == capi.E_NULL   # blocked weights carry no ldw
+    assert hb(0, 0, 8, 16, None, 16, None, 16, 0, None, None) == capi.OK
+    # the failing barrier of the single-launch decode forward is a test hook: refused without FSW_TEST_HOOKS=1
+    os.environ.pop("FSW_TEST_HOOKS", None)
+    assert L.fsw_set_variant(0, 103) == capi.E_VARIANT and L.fsw_set_variant(0, 101) == capi.OK
+    assert L.fsw_set_variant(0, -1) == capi.OK
     assert L.fsw_set_variant(7, 0) == capi.E_VARIANT
     assert L.fsw_set_variant(2, 4) == capi.E_VARIANT and L.fsw_set_variant(0, 6) == capi.E_VARIANT
     assert L.fsw_mlp(7, 4, 16, 8, 0x1000, 16, 0x2000, 16, 0x3000, 8, 0x4000, 16, None, 0, None) == capi.E_DTYPE
