@@ -147,7 +147,7 @@ int finish(hipError_t e) {
 
 extern "C" {
 
-int fsw_version(void) { return 1000; }
+int fsw_version(void) { return 2000; }
 
 const char* fsw_strerror(int code) {
   switch (code) {

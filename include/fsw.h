@@ -179,7 +179,8 @@ FSW_API int fsw_gateup_ws(int dtype, int64_t M, int64_t N, int64_t K, const void
 /* The hipError_t (as int) of the most recent failed launch on the calling thread, 0 if none. */
 FSW_API int fsw_last_hip_error(void);
 
-/* ABI version: major * 1000 + minor. */
+/* ABI version: major * 1000 + minor. 2000: the measurement kernels fsw_probe_* left this library (libfsw_probe.so,
+ * fsw_probe.h); fsw_gateup_f32out and fsw_gateup_hblocked joined it; fsw_gateup_workspace_bytes returns 0. */
 FSW_API int fsw_version(void);
 
 /*
