@@ -182,8 +182,13 @@ tiled_pair16_kernel(const GemmArgs a_in, const int tiles_p, const int tiles_q, c
       fr[set][idx - NB] = *(const u32x4*)(pslot + rd_p + p_block_off(idx - NB) + (PBLK ? 0u : xp[half]));
     }
   };
+  // MFMA i of a K tile: weight block f = i / 8, activation block g walking forth on even f and back on odd f, so
+  // that exactly one operand changes from any MFMA to the next (at the end of a row of blocks only the weight
+  // fragment). Operand register reads cost power like everything else here: against restarting g at 0 the whole
+  // forward at 8192 x 4096 x 14336 measures 0.5 % faster (1.8628 vs 1.8728 ms), bit-identical.
   auto mma_one = [&](int set, int i) {
-    E::mfma16_acc(acc[i / NB][i % NB], fr[set][i / NB], fr[set][NB + i % NB]);
+    const int f = i / NB, g = (f & 1) ? NB - 1 - i % NB : i % NB;
+    E::mfma16_acc(acc[f][g], fr[set][f], fr[set][NB + g]);
   };
   // activation copy j (0 .. 7) of pair `pair`: tile 2 pair + j / 4; tiles past the end arrive as zeros
   // (QROW: st_a is the pair slot, st_b unused; copy j covers rows 32 j .. 32 j + 31 of the pair, 128 bytes each)

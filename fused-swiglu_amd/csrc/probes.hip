@@ -35,7 +35,10 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(const u32x4* __restrict
 #pragma unroll
     for (int f = 0; f < 8; ++f)
 #pragma unroll
-      for (int g = 0; g < 8; ++g) E::mfma16_acc(acc[f][g], a[f], b[g]);
+      for (int gg = 0; gg < 8; ++gg) {  // the prefill kernel's order: one operand changes per MFMA
+        const int g = (f & 1) ? 7 - gg : gg;
+        E::mfma16_acc(acc[f][g], a[f], b[g]);
+      }
   }
   mfma_drain();
   float s = 0.f;
