@@ -101,6 +101,22 @@ int64_t decode_rows(int family, int64_t np, int64_t k) {
   return d_ff < ((int64_t)1 << 25) ? 48 : d_ff < ((int64_t)1 << 27) ? 32 : 16;
 }
 
+// Weight rows per workgroup of the 128-row tiled kernels when ONE tile of activation rows streams the whole weight
+// matrix (gate/up): cut into 128-row tiles a matrix of fewer than 256 x 128 rows leaves compute units idle, and one
+// compute unit fetches at most ~29 GB/s, so the stream is cut into one piece per compute unit instead (a multiple of 8
+// rows; the kernel's copies of the rows past its piece are out of range and cost no traffic). Gate/up alone, 128-row
+// tiles -> pieces, us: 16384 rows (128 tiles -> 256 x 64) M = 64 33.8 -> 31.0, M = 128 41.1 -> 39.3; 22016 rows (172 ->
+// 251 x 88) 36.1 -> 34.2, 43.4 -> 41.9; 27648 rows (216 -> 247 x 112) M = 16 47.0 -> 45.3, M = 64 52.0 -> 49.4, M = 128
+// 62.6 -> 60.0. Not with 224 tiles or more (28672 rows: 35.2 -> 35.8, the pieces' wasted MFMA and LDS work costs more
+// than the 32 idle compute units) and not above 128 activation rows, where the matrix cores are the limit (16384 rows,
+// M = 256: 53.5 -> 56.2). 0 = the kernel's own tile height.
+int stream_tile_rows(int variant, int64_t m, int64_t np) {
+  if (!(variant == V_128x64 && m <= 64) && !(variant == V_128x128 && m <= 128)) return 0;
+  if ((np + 127) / 128 > 216) return 0;
+  const int64_t rows = ((np + 255) / 256 + 7) / 8 * 8;
+  return (rows >= 64 && rows < 128) ? (int)rows : 0;
+}
+
 int resolve_variant(int family, int64_t m, int64_t np, int64_t k) {
   const int forced = g_forced_variant[family];
   if (forced == VARIANT_DECODE_FUSED || forced == VARIANT_DECODE_FUSED_FAIL || forced == VARIANT_DECODE_STREAM ||
@@ -270,6 +286,7 @@ static int gateup_impl(int dtype, int64_t M, int64_t N, int64_t K, const void* X
   a.zero_words = zero_words;
   a.n_zero_words = n_zero_words;
   const int v = resolve_variant(0, M, N, K);
+  a.tile_p = stream_tile_rows(v, M, N);
   if (v == VARIANT_SKINNY) {
     if (decode_stream_wanted(0, M, N, K)) {  // at most 16 rows: one 8-wave workgroup per CU, X held in registers
       fsw::DecodeArgs da = {};

@@ -31,6 +31,11 @@ struct GemmArgs {
   // gated kernels on row-major operands (skinny_kernel, the 256 x 256 kernel with layout 0): O is float [nq, np/2]
   // and receives the gated fp32 value unrounded (the reference's build with C_TYPE float, constants.cuh:9)
   int out_f32 = 0;
+  // tiled_dma_kernel with one tile of activation rows: weight rows a workgroup owns when that is fewer than the
+  // kernel's tile height (0 = the tile height). The tile then starts every tile_p rows, rows past tile_p are out
+  // of range for its copies (zeros, no traffic) and are not stored: lets a weight stream be cut into exactly as
+  // many pieces as there are compute units. A multiple of 8 (whole 8-byte stores of the gated output).
+  int tile_p = 0;
 };
 inline long long blocked_bytes(long long rows, long long k) {
   return ((rows + 255) / 256) * ((k + 31) / 32) * (256 * 64);

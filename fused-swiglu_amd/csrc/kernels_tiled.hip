@@ -26,9 +26,9 @@ namespace fsw {
 // 8-byte store.
 template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
 __device__ __forceinline__ void store_tile(f32x16 (&acc)[FP][FQ], const GemmArgs& a, int p0, int q0, int wp, int wq,
-                                           int l32, int hi) {
+                                           int l32, int hi, int p_end) {
   unsigned short* O = (unsigned short*)a.O;
-  const int nout = GATED ? a.np / 2 : a.np;
+  const int nout = GATED ? p_end / 2 : p_end;  // p_end: first weight row this workgroup does not own
   const bool vec_ok = ((a.ldo & 3) == 0) && ((((uintptr_t)a.O) & 7) == 0);
   constexpr int FO = GATED ? FP / 2 : FP;
 #pragma unroll
@@ -173,7 +173,9 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
 
   int tp, tq;
   tile_coords(blockIdx.x, tiles_p, tiles_q, group, tp, tq);
-  const int p0 = tp * BP;
+  const int step_p = (a.tile_p > 0 && a.tile_p < BP) ? a.tile_p : BP;  // weight rows this workgroup owns
+  const int p0 = tp * step_p;
+  const int p_end = p0 + step_p < a.np ? p0 + step_p : a.np;
   const int q0 = tq * BQ;
   if (GATED && blockIdx.x == 0 && blockIdx.y == 0)  // counters of the kernel that follows in fsw_mlp (GemmArgs::zero_words)
     for (int i = t; i < a.n_zero_words; i += NT) a.zero_words[i] = 0u;
@@ -184,7 +186,7 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
   const int lc = pc ^ ((rb >> 1) & 7);  // logical chunk this lane fetches (RSTEP % 16 == 0 keeps (row >> 1) & 7)
   const unsigned char* pbase = (const unsigned char*)a.P + (long long)p0 * a.ldp * 2;
   const unsigned char* qbase = (const unsigned char*)a.Q + (long long)q0 * a.ldq * 2;
-  const __amdgpu_buffer_rsrc_t prs = make_rsrc(pbase, ((long long)(a.np - p0 - 1) * a.ldp + a.k) * 2);
+  const __amdgpu_buffer_rsrc_t prs = make_rsrc(pbase, ((long long)(p_end - p0 - 1) * a.ldp + a.k) * 2);
   const __amdgpu_buffer_rsrc_t qrs = make_rsrc(qbase, ((long long)(a.nq - q0 - 1) * a.ldq + a.k) * 2);
   unsigned poff[LP], qoff[LQ];
 #pragma unroll
@@ -398,7 +400,7 @@ tiled_dma_kernel(const GemmArgs a, const int tiles_p, const int tiles_q, const i
       return;
     }
   }
-  store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi);
+  store_tile<E, GATED, WP, WQ, FP, FQ>(acc, a, p0, q0, wp, wq, l32, hi, p_end);
 }
 
 // ---- row-major -> panel-blocked copy ---------------------------------------------------------------------------
@@ -477,7 +479,8 @@ void launch_dma_kernel(const dim3 grid, hipStream_t stream, const GemmArgs& a, i
 template <class E, bool GATED, int WP, int WQ, int FP, int FQ>
 hipError_t launch_dma(const GemmArgs& a, hipStream_t stream) {
   constexpr int BP = WP * FP * 32, BQ = WQ * FQ * 32;
-  const int tiles_p = (a.np + BP - 1) / BP;
+  const int step_p = (a.tile_p > 0 && a.tile_p < BP) ? a.tile_p : BP;
+  const int tiles_p = (a.np + step_p - 1) / step_p;
   const int tiles_q = (a.nq + BQ - 1) / BQ;
   if (tiles_p <= 0 || tiles_q <= 0) return hipSuccess;
   const dim3 grid((unsigned)(tiles_p * tiles_q));

@@ -575,6 +575,42 @@ def test_swiglu_fwd_bf16_writes_dense_half_width_rows(ext):
         ext.swiglu_fwd_bf16(M, N + 1, K, g["X"], K, g["W13"], K, C, N)  # odd N
 
 
+@pytest.mark.parametrize("shape", [(16, 520, 8200), (64, 136, 11008), (128, 264, 13824), (100, 72, 8192), (40, 64, 10004)])
+def test_weight_stream_cut_into_one_piece_per_compute_unit(capi, shape):
+    """Gate/up with one tile of activation rows and between 128 and 216 tiles of 128 weight rows: the dispatcher hands
+    every workgroup a piece of 64 .. 120 rows instead (as many pieces as compute units), whose tile reads its missing
+    rows as zeros and stores only the features it owns. Against the oracle (every feature, so a piece that stored a
+    neighbour's features from its zero rows would show as zeros there) and against the kernel on whole 128-row tiles; H
+    inside a wider NaN buffer, so a store past the row's end would show."""
+    M, d, ff = shape
+    dtype = torch.bfloat16 if ff % 16 == 0 else torch.float16
+    inp = fsw_weights.make_inputs(M, d, ff, dtype, seed=M + ff, x_scale=0.5)
+    g = to_dev(inp)
+    want = "dma_128x64" if M <= 64 else "dma_128x128"
+    forced = capi.variant_name(0, 0, M, 2 * ff, d) != want  # small K: the weight-streaming kernel would run
+    wide = torch.full((M, ff + 8), float("nan"), dtype=dtype, device=DEV)
+    try:
+        if forced:
+            capi.set_variant(0, 4)
+        assert capi.variant_name(0, 0, M, 2 * ff, d) == want
+        H = capi.gateup(g["X"], g["W13"], out=wide[:, :ff])
+    finally:
+        capi.set_variant(0, -1)
+    assert_one_rounding(H, oracle.ref_gateup(inp["X"], inp["W13"], torch.float64), dtype, "pieces %s" % (shape,))
+    assert torch.isnan(wide[:, ff:]).all()
+    # the same kernel on whole tiles: a problem of the same rows that the rule leaves alone (more than 128 activation
+    # rows cannot be built from these, so force the unsplit 128 x 128 kernel on a row-padded X instead)
+    Xp = torch.zeros((129, d), dtype=dtype, device=DEV)
+    Xp[:M] = g["X"]
+    try:
+        capi.set_variant(0, 0)
+        Hp = capi.gateup(Xp, g["W13"])
+    finally:
+        capi.set_variant(0, -1)
+    # (not bit for bit: with one tile of activation rows every workgroup starts its K walk at its own K tile)
+    assert (Hp[:M].float() - H.float()).abs().max().item() <= 2 * ulp_rel(dtype) * H.float().abs().max().item() + 1e-3
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [1, 16, 64, 65, 300, 1024])
 def test_float32_output_is_the_unrounded_gated_value(capi, M, dtype):
