@@ -851,11 +851,12 @@ def test_mlp_large_tile_regime_uses_blocked_path(capi):
     assert torch.equal(Y4, capi.down(capi.gateup(g["X"], g["W13"]), g["W2"]))
 
 
-@pytest.mark.parametrize("shape", [(16, 512, 1024), (96, 512, 1024), (600, 1024, 520)])
+@pytest.mark.parametrize("shape", [(16, 512, 1024), (96, 512, 1024), (600, 1024, 520), (2304, 4096, 2048)])
 def test_forward_replays_from_a_hip_graph(capi, shape):
     """fsw_mlp enqueues kernels only (no allocation, no synchronisation, no memset), so a caller can capture it into a
     HIP graph. Every replay — with eager work and synchronisations of the program in between, and with new contents
-    in the input buffer — must reproduce the eager result bit for bit. Decode, mid and large-tile regimes."""
+    in the input buffer — must reproduce the eager result bit for bit. Decode, mid and large-tile regimes, the last
+    shape with H panel-blocked between the two kernels."""
     M, d, ff = shape
     inp = fsw_weights.make_inputs(M, d, ff, torch.bfloat16, seed=123, x_scale=0.5)
     g = to_dev(inp)
@@ -879,9 +880,9 @@ def test_forward_replays_from_a_hip_graph(capi, shape):
 
 
 def test_large_tiles_on_row_major_activations(capi):
-    """256 x 256 tiles with ROW-MAJOR activations: fsw_gateup for a ragged M below 1024 (no re-blocking there) and
-    fsw_down without the optional scratch for a blocked copy of H. Both against the oracle, and the down projection
-    bit for bit against the call that does get the scratch."""
+    """256 x 256 tiles with ROW-MAJOR activations (fetched in K pairs of one whole line per row): fsw_gateup for a
+    ragged M and a K that is no multiple of 64, fsw_down without any scratch. Both against the oracle, and the down
+    projection bit for bit against the blocked form of the same kernel (H re-blocked by fsw_block_rows first)."""
     L = capi.lib()
     M, d, ff = 1000, 520, 12800          # 4 x 100 tiles of 256 x 256, K = 520 is not a multiple of 64
     assert capi.variant_name(0, 0, M, 2 * ff, d) == "pair16_256x256" and L.fsw_gateup_workspace_bytes(0, M, 2 * ff, d) == 0
@@ -900,7 +901,8 @@ def test_large_tiles_on_row_major_activations(capi):
     Y0 = torch.empty(M2, D2, dtype=torch.float16, device=DEV)
     s = torch.cuda.current_stream().cuda_stream
     capi.check(L.fsw_down(1, M2, D2, FF2, Hd.data_ptr(), FF2, W2d.data_ptr(), FF2, Y0.data_ptr(), D2, None, 0, s))
-    Y1 = capi.down(Hd, W2d)               # with scratch: H re-blocked first
+    assert torch.equal(Y0, capi.down(Hd, W2d)) and L.fsw_down_workspace_bytes(1, M2, D2, FF2) == 0
+    Y1 = capi.down_blocked(capi.block_rows(Hd), W2d)   # the same products in the same K order from a blocked H
     assert torch.equal(Y0, Y1)
     rows = torch.arange(0, M2, 31)
     assert_one_rounding(Y0[rows.to(DEV)], Hh[rows].double() @ W2.double().T, torch.float16, "row-major H, 256x256")
