@@ -37,9 +37,10 @@ sys.path.insert(0, os.path.join(ROOT, "fused-swiglu_amd"))
 MFMA_PEAK_TFLOPS = 2516.6  # MI355X dense bf16/fp16: 256 CU x 2.4 GHz x 4096 flop/clk/CU
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 DECODE_WARMUP = 500        # untimed forwards before the HBM-bound (M = 16) measurements, ~30 ms
-SETTLE_MS = 60.0           # untimed forwards before the timed steps of the compute-bound legs, whatever --warmup says:
-                           # after an idle period the board's clock needs ~25 ms of load to settle (the reference's
-                           # timer, bench_swiglu.py:102-106, warms up for about as long)
+SETTLE_MS = 200.0          # untimed forwards before the timed steps of the compute-bound legs, whatever --warmup says:
+                           # after an idle period the board's clock needs ~50 ms of load to settle (the first 30
+                           # forwards run 10 % slower), and on some boxes the step time keeps falling by another
+                           # 0.5 % over the next 100 ms; the reference's timer (bench_swiglu.py:102-106) warms up too
 FLUSH_BYTES = 512 << 20    # written before every timed call of the per-configuration leg (Infinity Cache: 256 MB)
 # counter profiles (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measurable in-process) that hold the line
 # `traffic_bytes_per_launch = N` for the dominant kernel of a workload
