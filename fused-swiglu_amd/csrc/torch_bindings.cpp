@@ -140,7 +140,7 @@ Tensor fused_swiglu_mlp_typed(at::ScalarType want, Tensor const& X, Tensor const
   Tensor Y = at::empty({M, D}, X.options());
   const at::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(device_of(X));
   const int code = dtype_code(want);
-  // one call: H (and, for large problems, a blocked copy of X) live in this scratch, never as a tensor
+  // one call: H (panel-blocked for large problems) and the split-K partials live in this scratch, never as a tensor
   const size_t ws_bytes = fsw_mlp_workspace_bytes(code, M, D, FF);
   Tensor ws = at::empty({(int64_t)std::max<size_t>(ws_bytes, 16)}, X.options().dtype(at::kByte));
   const int rc = fsw_mlp(code, M, D, FF, X.data_ptr(), M > 1 ? X.stride(0) : D, W1W3.data_ptr(),

@@ -122,7 +122,7 @@ FSW_API int fsw_mlp(int dtype, int64_t M, int64_t D, int64_t FF,
 /*
  * fsw_mlp for callers that cannot allocate device memory at all (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): same arguments without the workspace, same kernels, same result bit for
- * bit. No counterpart in the reference. The scratch (H, split-K partials, the blocked copy of X) lives in a static
+ * bit. No counterpart in the reference. The scratch (H, split-K partials and their ticket counters) lives in a static
  * device array of fsw_mlp_static_max_bytes() = 64 MiB inside the library, which every GPU the library runs on holds
  * until the process ends; shapes whose fsw_mlp_workspace_bytes() exceed it return FSW_E_STATIC_LIMIT (it covers
  * decode and small batches: at d = 4096, ff = 14336 every M <= 468). The call itself allocates and frees nothing;
