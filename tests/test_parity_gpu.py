@@ -611,6 +611,22 @@ def test_weight_stream_cut_into_one_piece_per_compute_unit(capi, shape):
     assert (Hp[:M].float() - H.float()).abs().max().item() <= 2 * ulp_rel(dtype) * H.float().abs().max().item() + 1e-3
 
 
+def test_pieces_zero_the_ticket_counters_of_the_down_projection_too(capi):
+    """A decode-sized forward whose gate/up stream is cut into pieces (27648 rows: 247 pieces of 112) AND whose down
+    projection is the split-K streaming kernel (24 rows): the first workgroup of the gate/up launch still zeroes the
+    ticket counters, whatever rows it owns. Workspace full of garbage, repeated calls bit for bit."""
+    M, d, ff = 24, 5120, 13824
+    assert capi.variant_name(0, 0, M, 2 * ff, d) == "dma_128x64" and capi.variant_name(2, 0, M, d, ff) == "stream_split"
+    inp = fsw_weights.make_inputs(M, d, ff, torch.bfloat16, seed=61, x_scale=0.5)
+    g = to_dev(inp)
+    ws = capi.mlp_workspace(g["X"], ff)
+    ws.fill_(0xC3)
+    Y = capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws)
+    oracle.assert_parity(Y, oracle.ref_mlp(inp["X"], inp["W13"], inp["W2"], torch.float64), "pieces + stream_split")
+    for _ in range(5):
+        assert torch.equal(capi.mlp(g["X"], g["W13"], g["W2"], workspace=ws), Y)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M", [1, 16, 64, 65, 300, 1024])
 def test_float32_output_is_the_unrounded_gated_value(capi, M, dtype):
